@@ -1,0 +1,88 @@
+// Shared host/device helpers for the artk C-ABI library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/artk.h"
+
+namespace artk {
+
+// ---- error reporting (thread-local message, integer return codes) ----------
+void set_error(const char* fmt, ...);
+
+#define ARTK_CHECK_ARG(cond, ...)         \
+  do {                                    \
+    if (!(cond)) {                        \
+      artk::set_error(__VA_ARGS__);       \
+      return ARTK_ERR_INVALID_ARGUMENT;   \
+    }                                     \
+  } while (0)
+
+#define ARTK_CHECK_HIP(expr)                                                        \
+  do {                                                                              \
+    hipError_t e__ = (expr);                                                        \
+    if (e__ != hipSuccess) {                                                        \
+      artk::set_error("%s failed: %s", #expr, hipGetErrorString(e__));              \
+      return (int32_t)e__;                                                          \
+    }                                                                               \
+  } while (0)
+
+#define ARTK_CHECK_LAUNCH()                                                         \
+  do {                                                                              \
+    hipError_t e__ = hipGetLastError();                                             \
+    if (e__ != hipSuccess) {                                                        \
+      artk::set_error("kernel launch failed at %s:%d: %s", __FILE__, __LINE__,      \
+                      hipGetErrorString(e__));                                      \
+      return (int32_t)e__;                                                          \
+    }                                                                               \
+  } while (0)
+
+static inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Bump allocator over a caller-provided workspace.
+struct Workspace {
+  char* base;
+  size_t size;
+  size_t used;
+  Workspace(void* p, size_t n) : base((char*)p), size(n), used(0) {}
+  // Returns nullptr when the workspace is exhausted (or absent while sizing).
+  template <typename T>
+  T* take(size_t count) {
+    size_t off = align_up(used, 256);
+    used = off + count * sizeof(T);
+    if (base == nullptr || used > size) return nullptr;
+    return (T*)(base + off);
+  }
+  bool ok() const { return base != nullptr && used <= size; }
+};
+
+// ---- device helpers ---------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  __bf16 h = (__bf16)f;  // round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
+  return __builtin_bit_cast(uint16_t, h);
+}
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+}  // namespace artk

@@ -1,0 +1,219 @@
+// NT bf16 GEMM main loop for gfx950 (MI355X, CDNA4).
+//
+// Computes a 256x256 tile of  C[i][j] = sum_k P[i][k] * Q[j][k]  where both
+// operands are row-major with K contiguous ("NT").  P is the "row operand"
+// (its row index ends up in the accumulator registers of a lane), Q is the
+// "column operand" (its row index is the lane's column).  The callers put the
+// matrix whose row index is the *contiguous* dimension of the output into the
+// P role, so that each lane owns 4 consecutive output elements.
+//
+// Work-group: 256 threads = 4 wavefronts (64 lanes) in a 2x2 grid, each
+// wavefront owns a 128x128 sub-tile = 4x4 MFMA 32x32x16 bf16 tiles, i.e. 256
+// fp32 accumulator registers per lane.  One work-group per CU (1 wave / SIMD).
+//
+// Data path: HBM/L2 -> LDS by buffer_load_dwordx4 ... lds (no VGPR staging),
+// two LDS stages of 2 x 32 KiB, 16-byte chunks XOR-swizzled so that both the
+// DMA writes (1 KiB contiguous per wave instruction) and the ds_read_b128
+// operand reads are bank-conflict free.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace artk {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+constexpr int TILE = 256;       // tile rows of either operand
+constexpr int BK = 64;          // K elements per LDS stage
+constexpr int NTHREADS = 256;   // 4 wavefronts
+constexpr int OPER_STAGE_BYTES = TILE * BK * 2;          // 32 KiB
+constexpr int STAGE_BYTES = 2 * OPER_STAGE_BYTES;         // P + Q
+constexpr int NSTAGES = 2;
+constexpr int GEMM_LDS_BYTES = NSTAGES * STAGE_BYTES;     // 128 KiB
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Swizzle of the 16-byte chunk index within a 128-byte LDS row.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// One operand of the NT GEMM as seen by one wavefront's DMA instructions.
+struct OperandLoader {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int voff[8];  // per-lane byte offset of the 8 DMA instructions of this wave
+
+  // base: first element of the operand; ld: leading dimension in elements;
+  // row0: first tile row; nrows: rows the operand really has (rows past the
+  // end are clamped to the last valid row; the epilogue never stores them).
+  __device__ __forceinline__ void init(const void* base, int64_t ld, int64_t row0,
+                                       int64_t nrows, int wave, int lane) {
+    const char* p = (const char*)base + row0 * ld * 2;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
+    int64_t left = nrows - row0;
+    int nvalid = left >= TILE ? TILE : (int)left;
+    int r = lane >> 3, pc = lane & 7;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int row = (wave * 8 + i) * 8 + r;
+      int kc = pc ^ swz(row);
+      int rc = row < nvalid ? row : nvalid - 1;
+      voff[i] = (int)(rc * ld * 2) + kc * 16;
+    }
+  }
+
+  // Issue this wave's 8 DMA instructions for K offset k0 (elements) into the
+  // 32 KiB operand stage at `stage` (LDS byte address, wave-uniform).
+  __device__ __forceinline__ void issue(char* stage, int wave, int k0) const {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * 8 + i) * 1024), 16,
+                                               voff[i], k0 * 2, 0, 0);
+    }
+  }
+};
+
+struct TileAcc {
+  floatx16 c[4][4];  // [mi][ni]
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) c[mi][ni][j] = 0.f;
+  }
+};
+
+// Row (P-operand index, tile-relative) of accumulator element j of MFMA tile mi
+// for this lane, and column (Q-operand index, tile-relative) of MFMA tile ni.
+__device__ __forceinline__ int acc_row(int wm, int mi, int j, int lane) {
+  return wm * 128 + mi * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+}
+__device__ __forceinline__ int acc_col(int wn, int ni, int lane) {
+  return wn * 128 + ni * 32 + (lane & 31);
+}
+
+// Operand fragments of one K=16 step: 4 row-operand and 4 column-operand reads.
+struct Frags {
+  bf16x8 p[4], q[4];
+};
+
+__device__ __forceinline__ void load_frags(Frags& f, const char* sp, const char* sq, int off) {
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) f.p[mi] = *(const bf16x8*)(sp + off + mi * 4096);
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) f.q[ni] = *(const bf16x8*)(sq + off + ni * 4096);
+}
+
+__device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni)
+      acc.c[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.p[mi], f.q[ni], acc.c[mi][ni], 0, 0, 0);
+}
+
+// Main loop: acc += P[prow0 : prow0+256, k_begin : k_end] * Q[qrow0 : qrow0+256, same]^T.
+// k_begin/k_end are multiples of BK, k_end > k_begin.  `smem` is GEMM_LDS_BYTES
+// of LDS, 1 KiB aligned.
+//
+// Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 16 MFMAs each):
+//   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read
+//   wait for own LDS reads and own DMA, barrier:
+//                every wave holds its step-3 fragments in registers, so the
+//                current stage is free, and the next stage has landed
+//   DMA for the stage after next goes into the freed buffer
+//   step 3     : MFMAs while step 0 of the next stage is read
+// The loop body has no branches: past the end, the DMA re-fetches the last
+// stage into the idle buffer and the fragment prefetch reads values nobody uses.
+__device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const void* P, int64_t ldp,
+                                             int64_t prow0, int64_t prows, const void* Q,
+                                             int64_t ldq, int64_t qrow0, int64_t qrows, int k_begin,
+                                             int k_end) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  OperandLoader lp, lq;
+  lp.init(P, ldp, prow0, prows, wave, lane);
+  lq.init(Q, ldq, qrow0, qrows, wave, lane);
+
+  // Per-lane LDS read offsets (within an operand stage) for the 4 K=16 steps.
+  int off[4];
+  {
+    int rl = lane & 31;
+    int f = swz(rl);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) off[kk] = rl * 128 + (((kk * 2 + (lane >> 5)) ^ f) << 4);
+  }
+  const int p_wave_off = wm * 128 * 128;
+  const int q_wave_off = OPER_STAGE_BYTES + wn * 128 * 128;
+
+  const int nk = (k_end - k_begin) / BK;
+  const int k_last = k_end - BK;
+
+  lp.issue(smem, wave, k_begin);
+  lq.issue(smem + OPER_STAGE_BYTES, wave, k_begin);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  {
+    int k1 = k_begin + BK < k_last ? k_begin + BK : k_last;
+    lp.issue(smem + STAGE_BYTES, wave, k1);
+    lq.issue(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
+  }
+  Frags f0, f1;
+  load_frags(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    char* cur = smem + (kt & 1) * STAGE_BYTES;
+    char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
+    const char* sp = cur + p_wave_off;
+    const char* sq = cur + q_wave_off;
+
+    load_frags(f1, sp, sq, off[1]);
+    mma_frags(acc, f0);
+    load_frags(f0, sp, sq, off[2]);
+    mma_frags(acc, f1);
+    load_frags(f1, sp, sq, off[3]);
+    mma_frags(acc, f0);
+#pragma unroll
+    for (int i = 0; i < 24; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+    }
+
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    int k2 = k_begin + (kt + 2) * BK;
+    k2 = k2 < k_last ? k2 : k_last;
+    lp.issue(cur, wave, k2);
+    lq.issue(cur + OPER_STAGE_BYTES, wave, k2);
+    load_frags(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
+    mma_frags(acc, f1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // 2 DMA issues
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+    }
+  }
+  // Drain the redundant tail DMA before the caller reuses or releases LDS.
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+}
+
+// Map the hardware's round-robin block->XCD placement (block b runs on XCD
+// b % 8) onto contiguous ranges of logical tile ids, so that tiles sharing
+// operand panels run on the same XCD and hit in its private L2.
+__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
+  int full = nblocks >> 3, rem = nblocks & 7;
+  int x = bid & 7, loc = bid >> 3;
+  int start = x * full + (x < rem ? x : rem);
+  return start + loc;
+}
+
+}  // namespace artk

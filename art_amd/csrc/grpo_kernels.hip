@@ -1,0 +1,882 @@
+// GRPO logprob / loss hot path for gfx950: lm_head projection with online
+// log-sum-exp and target gather, clipped-surrogate loss with its gradient
+// coefficient, softmax gradient and the d_hidden GEMM.
+//
+// Reference behaviour that these kernels restate:
+//   src/art/local/train.py:245-281  chunked matmul -> gather -> logsumexp
+//   src/art/local/train.py:284-285  shift_tensor (folded into index math here)
+//   src/art/local/train.py:111-151  ratio / clip / KL / weight*mask / normalise
+#include "common.hpp"
+#include "gemm_nt.hpp"
+
+#include <math.h>
+
+namespace artk {
+
+// ----------------------------------------------------------------------------
+// index helpers
+// ----------------------------------------------------------------------------
+
+// Element of a per-token input seen by position t: with shift, element t+1 of
+// the same row of the [B,S] input, or the pad value at the row's last position.
+__device__ __forceinline__ bool shifted_index(int64_t t, int64_t S, int shift, int64_t& src) {
+  if (!shift) {
+    src = t;
+    return true;
+  }
+  int64_t s = t % S;
+  src = t + 1;
+  return s + 1 < S;
+}
+
+__device__ __forceinline__ int64_t target_id(const int64_t* ids, int64_t t, int64_t S, int shift) {
+  int64_t src;
+  return shifted_index(t, S, shift, src) ? ids[src] : (int64_t)0;  // pad id 0 (train.py:79)
+}
+
+// ----------------------------------------------------------------------------
+// K1: logits tile = lm_head[256 vocab rows] x hidden[256 positions]^T, with
+// per-position (max, sum-exp) partials over the tile's vocab rows, gather of
+// the target logit, and (optionally) the bf16 logits stored to a scratch.
+// ----------------------------------------------------------------------------
+struct FwdParams {
+  const void* hidden;   // [Tc,H] bf16: first row = position t0
+  const void* W;        // [V,H] bf16
+  const int64_t* ids;   // [T] (whole batch)
+  int64_t t0, Tc, T, S, V, H;
+  int shift;
+  float2* part;         // [2*VT][Tc]  (max, sumexp)
+  float* sel;           // [Tc]        selected logit (pre-filled with NaN)
+  uint16_t* stash;      // [Tc,V] bf16 logits or nullptr
+  int VT, TT;
+};
+
+template <bool STASH>
+__global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vt = id / p.TT, tt = id % p.TT;
+
+  TileAcc acc;
+  acc.zero();
+  gemm_tile_nt(acc, smem, p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE,
+               p.Tc, 0, (int)p.H);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+  const int64_t vbase = (int64_t)vt * TILE + wm * 128;  // first vocab row of this wave
+
+  // Targets of this lane's 4 positions (issued early: consumed after the reductions).
+  int64_t y[4];
+  int col[4];
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    col[ni] = tt * TILE + acc_col(wn, ni, lane);
+    y[ni] = col[ni] < p.Tc ? target_id(p.ids, p.t0 + col[ni], p.S, p.shift) : (int64_t)-1;
+  }
+
+  if (STASH) {
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      if (col[ni] < p.Tc) {
+        uint16_t* row = p.stash + (int64_t)col[ni] * p.V;
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            int64_t v = vbase + mi * 32 + q * 8 + half * 4;
+            if (v < p.V) {
+              bf16x4 o;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
+              *(bf16x4*)(row + v) = o;
+            }
+          }
+      }
+    }
+  }
+
+  // Vocab rows past V (last tile only) must not enter the reductions.
+  if ((int64_t)vt * TILE + TILE > p.V) {
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        int64_t v = vbase + mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+        if (v >= p.V) {
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) acc.c[mi][ni][j] = -INFINITY;
+        }
+      }
+  }
+
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    // A position's 128 logits of this wave: 64 in this lane, 64 in lane^32.
+    float m = -INFINITY;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) m = fmaxf(m, acc.c[mi][ni][j]);
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    const float mb = (m == -INFINITY ? 0.f : m) * LOG2E;
+    float l = 0.f;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        l += __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][j], LOG2E, -mb));
+    l += __shfl_xor(l, 32, 64);
+    if (lane < 32 && col[ni] < p.Tc)
+      p.part[(int64_t)(vt * 2 + wm) * p.Tc + col[ni]] = make_float2(m, l);
+
+    // Gather: exactly one lane of one wave of the whole grid holds logit[y].
+    const int64_t rel = y[ni] - vbase;
+    const bool hit = rel >= 0 && rel < 128 && ((((int)rel) >> 2) & 1) == half;
+    if (__any(hit)) {
+      float s = 0.f;
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+          if (r == (int)rel) s = acc.c[mi][ni][j];
+        }
+      if (hit) p.sel[col[ni]] = s;
+    }
+  }
+}
+
+// K2: merge the per-tile (max, sumexp) partials of each position.
+__global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restrict__ part,
+                                                           int nparts, int64_t Tc,
+                                                           const float* __restrict__ sel,
+                                                           float* __restrict__ logprob,
+                                                           float* __restrict__ lse) {
+  int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= Tc) return;
+  float M = -INFINITY;
+  for (int i = 0; i < nparts; ++i) M = fmaxf(M, part[(int64_t)i * Tc + t].x);
+  float L = 0.f;
+  for (int i = 0; i < nparts; ++i) {
+    float2 v = part[(int64_t)i * Tc + t];
+    L += v.y * __builtin_amdgcn_exp2f((v.x - M) * LOG2E);
+  }
+  float z = M + logf(L);
+  lse[t] = z;
+  logprob[t] = sel[t] - z;
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// ----------------------------------------------------------------------------
+// Loss kernels
+// ----------------------------------------------------------------------------
+
+// Number of positions whose (shifted) assistant mask is set. One block.
+__global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restrict__ mask,
+                                                          int64_t T, int64_t S, int shift,
+                                                          int* __restrict__ count) {
+  __shared__ int red[16];
+  int c = 0;
+  for (int64_t t = threadIdx.x; t < T; t += 1024) {
+    int64_t src;
+    if (shifted_index(t, S, shift, src)) c += mask[src] != 0;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int i = 0; i < 16; ++i) s += red[i];
+    *count = s;
+  }
+}
+
+struct LossParams {
+  const float* new_lp;   // [n] position frame, first element = position t0
+  const float* old_lp;   // [T] whole batch (frame given by shift)
+  const float* adv;      // [T]
+  const uint8_t* mask;   // [T]
+  const float* weights;  // [T]
+  const float* ref_lp;   // [n] position frame (same origin as new_lp) or nullptr
+  const int* count;      // mask count of the whole batch
+  int64_t t0, n, T, S;
+  int shift;
+  float clip_lo, clip_hi, beta;
+  float* pl_tok;         // [n] weighted policy-loss term
+  float* kl_tok;         // [n] weighted KL term
+  float* coef;           // [n] d loss / d new_lp, or nullptr
+};
+
+__global__ __launch_bounds__(256) void grpo_loss_tok_kernel(LossParams p) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= p.n) return;
+  const int64_t t = p.t0 + i;
+  int64_t src;
+  const bool in = shifted_index(t, p.S, p.shift, src);
+  float oldv = in ? p.old_lp[src] : 0.f;
+  const float adv = in ? p.adv[src] : 0.f;
+  const float w = in ? p.weights[src] : 0.f;
+  const float m = (in && p.mask[src] != 0) ? 1.f : 0.f;
+  const float nw = p.new_lp[i];
+  if (isnan(oldv)) oldv = nw;  // missing old logprob: sampled under the current policy
+  const float ratio = expf(nw - oldv);
+  const float a = ratio * adv;
+  const float clipped = fminf(fmaxf(ratio, p.clip_lo), p.clip_hi);
+  const float b = clipped * adv;
+  const float pl = -fminf(a, b);
+  // Gradient of -min(a, b) w.r.t. new_lp. Inside the clip range a and b are the
+  // same number and both pass the gradient; outside only a does, when it is the min.
+  const bool inside = ratio >= p.clip_lo && ratio <= p.clip_hi;
+  float g = (inside || a < b) ? -a : 0.f;
+  float kl = 0.f;
+  if (p.ref_lp != nullptr) {
+    const float d = p.ref_lp[i] - nw;
+    const float e = expf(d);
+    kl = e - d - 1.f;
+    g += p.beta * (1.f - e);
+  }
+  const float denom = (float)(*p.count) + 1e-6f;
+  const float wm = w * m;
+  p.pl_tok[i] = pl * wm;
+  p.kl_tok[i] = kl * wm;
+  if (p.coef) p.coef[i] = (wm != 0.f) ? g * wm / denom : 0.f;
+}
+
+// scalars = {loss, mean_policy_loss, mean_kl, mask_count}. One block; fixed
+// summation order, so the result is bit-reproducible run to run.
+__global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __restrict__ pl_tok,
+                                                                const float* __restrict__ kl_tok,
+                                                                int64_t T,
+                                                                const int* __restrict__ count,
+                                                                float beta,
+                                                                float* __restrict__ scalars) {
+  __shared__ double red[2][16];
+  double a = 0.0, b = 0.0;
+  for (int64_t t = threadIdx.x; t < T; t += 1024) {
+    a += (double)pl_tok[t];
+    b += (double)kl_tok[t];
+  }
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = a;
+    red[1][threadIdx.x >> 6] = b;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double sa = 0.0, sb = 0.0;
+    for (int i = 0; i < 16; ++i) {
+      sa += red[0][i];
+      sb += red[1][i];
+    }
+    const float denom = (float)(*count) + 1e-6f;
+    const float mpl = (float)sa / denom;
+    const float mkl = (float)sb / denom;
+    scalars[0] = mpl + beta * mkl;
+    scalars[1] = mpl;
+    scalars[2] = mkl;
+    scalars[3] = (float)(*count);
+  }
+}
+
+// ----------------------------------------------------------------------------
+// K3: in-place softmax gradient on the bf16 logits scratch:
+//   P[t,v] = coef[t] * ( [v == y_t] - exp(z[t,v] - lse[t]) )
+// One block per position; rows with coef == 0 are zero-filled without a read.
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict__ stash, int64_t V,
+                                                           const float* __restrict__ lse,
+                                                           const float* __restrict__ coef,
+                                                           const int64_t* __restrict__ ids,
+                                                           int64_t t0, int64_t S, int shift) {
+  const int64_t r = blockIdx.x;
+  uint4* row = (uint4*)(stash + r * V);
+  const int nvec = (int)(V >> 3);
+  const float c = coef[r];
+  if (c == 0.f) {
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (int i = threadIdx.x; i < nvec; i += 256) row[i] = z;
+    return;
+  }
+  const int64_t y = target_id(ids, t0 + r, S, shift);
+  const float nl = -lse[r] * LOG2E;
+  for (int i = threadIdx.x; i < nvec; i += 256) {
+    uint4 x = row[i];
+    uint32_t w[4] = {x.x, x.y, x.z, x.w};
+    const int64_t v0 = (int64_t)i * 8;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float z0 = __uint_as_float(w[e] << 16);
+      float z1 = __uint_as_float(w[e] & 0xffff0000u);
+      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(z0, LOG2E, nl));
+      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(z1, LOG2E, nl));
+      float g0 = c * ((v0 + 2 * e == y ? 1.f : 0.f) - p0);
+      float g1 = c * ((v0 + 2 * e + 1 == y ? 1.f : 0.f) - p1);
+      w[e] = (uint32_t)f32_to_bf16(g0) | ((uint32_t)f32_to_bf16(g1) << 16);
+    }
+    row[i] = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+// ----------------------------------------------------------------------------
+// K4: d_hidden tile = P[256 positions, k-range of V] x lm_head_t[256 h, same]^T
+// ----------------------------------------------------------------------------
+struct BwdParams {
+  const void* Wt;    // [H,V] bf16
+  const void* P;     // [Tc,V] bf16
+  int64_t V, H, Tc;
+  int nsplit, HT, TT;
+  float* partial;    // [nsplit][Tc][H] when nsplit > 1
+  uint16_t* out;     // [Tc,H] bf16 when nsplit == 1
+};
+
+__global__ __launch_bounds__(NTHREADS) void dhidden_gemm_kernel(BwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tiles = p.HT * p.TT;
+  const int split = id / tiles;
+  const int rem = id - split * tiles;
+  const int ht = rem / p.TT, tt = rem % p.TT;
+  const int KT = (int)(p.V / BK);
+  const int kb = (int)((int64_t)split * KT / p.nsplit);
+  const int ke = (int)((int64_t)(split + 1) * KT / p.nsplit);
+
+  TileAcc acc;
+  acc.zero();
+  gemm_tile_nt(acc, smem, p.Wt, p.V, (int64_t)ht * TILE, p.H, p.P, p.V, (int64_t)tt * TILE, p.Tc,
+               kb * BK, ke * BK);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    const int col = tt * TILE + acc_col(wn, ni, lane);
+    if (col >= p.Tc) continue;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t h = (int64_t)ht * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
+        if (h >= p.H) continue;
+        if (p.nsplit == 1) {
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
+          *(bf16x4*)(p.out + (int64_t)col * p.H + h) = o;
+        } else {
+          floatx4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = acc.c[mi][ni][q * 4 + e];
+          *(floatx4*)(p.partial + ((int64_t)split * p.Tc + col) * p.H + h) = o;
+        }
+      }
+  }
+}
+
+// K5: out = bf16(sum over splits of partial), 4 elements per thread.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
+                                                            int nsplit, int64_t n4,
+                                                            uint16_t* __restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  floatx4 s = ((const floatx4*)partial)[i];
+  for (int k = 1; k < nsplit; ++k) {
+    floatx4 v = ((const floatx4*)partial)[(int64_t)k * n4 + i];
+    s += v;
+  }
+  bf16x4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = (__bf16)s[e];
+  ((bf16x4*)out)[i] = o;
+}
+
+// ----------------------------------------------------------------------------
+// Transpose and plain GEMM
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ in,
+                                                             uint16_t* __restrict__ out, int64_t R,
+                                                             int64_t C) {
+  __shared__ uint16_t tile[64][66];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    int64_t r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? in[r * C + c] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int64_t c = c0 + i, r = r0 + tx;
+    if (c < C && r < R) out[c * R + r] = tile[tx][i];
+  }
+}
+
+struct GemmParams {
+  const void* P;
+  const void* Q;
+  void* out;
+  int64_t M, N, K;
+  int MT, NT, out_f32;
+};
+
+__global__ __launch_bounds__(NTHREADS) void gemm_nt_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int id = xcd_remap(blockIdx.x, gridDim.x);
+  const int mt = id / p.NT, nt = id % p.NT;
+  TileAcc acc;
+  acc.zero();
+  gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
+               (int)p.K);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    const int64_t col = (int64_t)nt * TILE + acc_col(wn, ni, lane);
+    if (col >= p.N) continue;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
+        if (m >= p.M) continue;
+        if (p.out_f32) {
+          floatx4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = acc.c[mi][ni][q * 4 + e];
+          *(floatx4*)((float*)p.out + col * p.M + m) = o;
+        } else {
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
+          *(bf16x4*)((uint16_t*)p.out + col * p.M + m) = o;
+        }
+      }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// Host side
+// ----------------------------------------------------------------------------
+static int num_cus() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
+// Split count for the d_hidden GEMM: fill whole rounds of CUs, keep every split
+// at least 32 K-steps long, prefer fewer splits on ties.
+static int choose_nsplit(int tiles, int ksteps) {
+  const int cus = num_cus();
+  int best = 1;
+  double best_eff = 0.0;
+  for (int ns = 1; ns <= 16; ++ns) {
+    if (ksteps / ns < 32 && ns > 1) break;
+    int blocks = tiles * ns;
+    int rounds = (blocks + cus - 1) / cus;
+    double eff = (double)blocks / ((double)rounds * cus);
+    if (eff > best_eff + 0.02) {
+      best_eff = eff;
+      best = ns;
+    }
+  }
+  return best;
+}
+
+static int32_t check_common(const void* hidden, const void* lm_head, int64_t T, int64_t S,
+                            int64_t V, int64_t H, bool need_v64) {
+  ARTK_CHECK_ARG(hidden && lm_head, "null hidden or lm_head pointer");
+  ARTK_CHECK_ARG(aligned16(hidden) && aligned16(lm_head), "hidden and lm_head must be 16-byte aligned");
+  ARTK_CHECK_ARG(T > 0 && S > 0 && V > 0 && H > 0, "T, S, V, H must be positive");
+  ARTK_CHECK_ARG(T % S == 0, "T (%lld) must be a multiple of the row length S (%lld)", (long long)T,
+                 (long long)S);
+  if (H % BK != 0) {
+    set_error("hidden size %lld must be a multiple of %d", (long long)H, BK);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  if (V % 8 != 0 || (need_v64 && V % BK != 0)) {
+    set_error("vocab size %lld must be a multiple of %d", (long long)V, need_v64 ? BK : 8);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  if (T >= (1ll << 31) / 4 || V >= (1ll << 31) / 512) {
+    set_error("T or V too large");
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  return ARTK_OK;
+}
+
+// Launch K1 (+ NaN pre-fill of sel) and K2 for positions [t0, t0+Tc).
+static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const int64_t* ids,
+                                int shift, int64_t t0, int64_t Tc, int64_t T, int64_t S, int64_t V,
+                                int64_t H, float2* part, float* sel, uint16_t* stash,
+                                float* logprob_chunk, float* lse_chunk, hipStream_t st) {
+  FwdParams p;
+  p.hidden = (const char*)hidden + t0 * H * 2;
+  p.W = lm_head;
+  p.ids = ids;
+  p.t0 = t0;
+  p.Tc = Tc;
+  p.T = T;
+  p.S = S;
+  p.V = V;
+  p.H = H;
+  p.shift = shift;
+  p.part = part;
+  p.sel = sel;
+  p.stash = stash;
+  p.VT = (int)((V + TILE - 1) / TILE);
+  p.TT = (int)((Tc + TILE - 1) / TILE);
+  fill_f32_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(sel, Tc, NAN);
+  ARTK_CHECK_LAUNCH();
+  const unsigned grid = (unsigned)(p.VT * p.TT);
+  if (stash)
+    lmhead_fwd_kernel<true><<<grid, NTHREADS, 0, st>>>(p);
+  else
+    lmhead_fwd_kernel<false><<<grid, NTHREADS, 0, st>>>(p);
+  ARTK_CHECK_LAUNCH();
+  lse_finalize_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
+                                                                    logprob_chunk, lse_chunk);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+// Launch K3, K4 (+K5) for one chunk whose bf16 logits are in `stash`.
+static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const int64_t* ids,
+                                int shift, int64_t t0, int64_t Tc, int64_t S, int64_t V, int64_t H,
+                                const float* lse_chunk, const float* coef_chunk, float* partial,
+                                int nsplit, uint16_t* d_hidden_chunk, hipStream_t st) {
+  softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, t0, S,
+                                                    shift);
+  ARTK_CHECK_LAUNCH();
+  BwdParams b;
+  b.Wt = lm_head_t;
+  b.P = stash;
+  b.V = V;
+  b.H = H;
+  b.Tc = Tc;
+  b.nsplit = nsplit;
+  b.HT = (int)((H + TILE - 1) / TILE);
+  b.TT = (int)((Tc + TILE - 1) / TILE);
+  b.partial = partial;
+  b.out = d_hidden_chunk;
+  dhidden_gemm_kernel<<<(unsigned)(b.HT * b.TT * nsplit), NTHREADS, 0, st>>>(b);
+  ARTK_CHECK_LAUNCH();
+  if (nsplit > 1) {
+    const int64_t n4 = Tc * H / 4;
+    splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(partial, nsplit, n4,
+                                                                       d_hidden_chunk);
+    ARTK_CHECK_LAUNCH();
+  }
+  return ARTK_OK;
+}
+
+static int bwd_nsplit(int64_t Tc, int64_t H, int64_t V) {
+  int tiles = (int)(((H + TILE - 1) / TILE) * ((Tc + TILE - 1) / TILE));
+  return choose_nsplit(tiles, (int)(V / BK));
+}
+
+// Split count for a chunk of n <= Tc positions that must fit the fp32 partial
+// buffer sized for `nsplit` splits of Tc positions.
+static int chunk_nsplit(int64_t n, int64_t Tc, int nsplit, int64_t H, int64_t V) {
+  if (nsplit <= 1) return 1;
+  if (n == Tc) return nsplit;
+  int ns = bwd_nsplit(n, H, V);
+  while (ns > 1 && (int64_t)ns * n > (int64_t)nsplit * Tc) --ns;
+  return ns;
+}
+
+}  // namespace artk
+
+using namespace artk;
+
+extern "C" {
+
+size_t artk_logprob_fwd_workspace_bytes(int64_t T, int64_t V, int64_t H) {
+  (void)H;
+  Workspace ws(nullptr, 0);
+  int64_t VT = (V + TILE - 1) / TILE;
+  ws.take<float2>((size_t)(2 * VT * T));
+  ws.take<float>((size_t)T);
+  return ws.used + 256;
+}
+
+int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t* ids, int32_t shift,
+                         int64_t T, int64_t S, int64_t V, int64_t H, float* logprob, float* lse,
+                         void* workspace, size_t workspace_bytes, artk_stream_t stream) {
+  int32_t rc = check_common(hidden, lm_head, T, S, V, H, false);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(ids && logprob && lse, "null ids/logprob/lse pointer");
+  ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
+  Workspace ws(workspace, workspace_bytes);
+  int64_t VT = (V + TILE - 1) / TILE;
+  float2* part = ws.take<float2>((size_t)(2 * VT * T));
+  float* sel = ws.take<float>((size_t)T);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  return launch_fwd_chunk(hidden, lm_head, ids, shift, 0, T, T, S, V, H, part, sel, nullptr, logprob,
+                          lse, (hipStream_t)stream);
+}
+
+static size_t chunk_workspace(int64_t T, int64_t V, int64_t H, int64_t Tc, bool with_loss,
+                              Workspace& ws, uint16_t** stash, float2** part, float** sel,
+                              float** partial, int* nsplit, float** lse, float** coef, float** pl,
+                              float** kl, int** count) {
+  int64_t VT = (V + TILE - 1) / TILE;
+  *stash = ws.take<uint16_t>((size_t)(Tc * V));
+  *part = ws.take<float2>((size_t)(2 * VT * Tc));
+  *sel = ws.take<float>((size_t)Tc);
+  *nsplit = bwd_nsplit(Tc, H, V);
+  *partial = *nsplit > 1 ? ws.take<float>((size_t)(*nsplit) * Tc * H) : nullptr;
+  if (with_loss) {
+    *lse = ws.take<float>((size_t)T);
+    *coef = ws.take<float>((size_t)T);
+    *pl = ws.take<float>((size_t)T);
+    *kl = ws.take<float>((size_t)T);
+    *count = ws.take<int>(64);
+  }
+  return ws.used + 256;
+}
+
+static int64_t clamp_chunk(int64_t T, int64_t chunk_tokens) {
+  if (chunk_tokens <= 0) chunk_tokens = 4096;
+  if (chunk_tokens > T) chunk_tokens = T;
+  return chunk_tokens;
+}
+
+size_t artk_logprob_bwd_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {
+  Workspace ws(nullptr, 0);
+  uint16_t* stash;
+  float2* part;
+  float *sel, *partial, *lse, *coef, *pl, *kl;
+  int nsplit, *count;
+  int64_t Tc = clamp_chunk(T, chunk_tokens);
+  size_t n = chunk_workspace(T, V, H, Tc, false, ws, &stash, &part, &sel, &partial, &nsplit, &lse,
+                             &coef, &pl, &kl, &count);
+  // scratch logprob / lse outputs of the recompute pass
+  return n + 2 * align_up((size_t)Tc * 4, 256) + 512;
+}
+
+int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm_head_t,
+                         const int64_t* ids, int32_t shift, int64_t T, int64_t S, int64_t V,
+                         int64_t H, const float* lse, const float* grad_logprob, void* d_hidden,
+                         int64_t chunk_tokens, void* workspace, size_t workspace_bytes,
+                         artk_stream_t stream) {
+  int32_t rc = check_common(hidden, lm_head, T, S, V, H, true);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(lm_head_t && ids && lse && grad_logprob && d_hidden, "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(lm_head_t) && aligned16(d_hidden), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
+  const int64_t Tc = clamp_chunk(T, chunk_tokens);
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* stash;
+  float2* part;
+  float *sel, *partial, *lse_u, *coef_u, *pl_u, *kl_u;
+  int nsplit, *count_u;
+  chunk_workspace(T, V, H, Tc, false, ws, &stash, &part, &sel, &partial, &nsplit, &lse_u, &coef_u,
+                  &pl_u, &kl_u, &count_u);
+  float* lp_tmp = ws.take<float>((size_t)Tc);
+  float* lse_tmp = ws.take<float>((size_t)Tc);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
+    const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
+    // The stash row pitch is V, so a shorter last chunk simply uses fewer rows.
+    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, t0, n, T, S, V, H, part, sel, stash, lp_tmp,
+                          lse_tmp, st);
+    if (rc) return rc;
+    rc = launch_bwd_chunk(stash, lm_head_t, ids, shift, t0, n, S, V, H, lse + t0, grad_logprob + t0,
+                          partial, chunk_nsplit(n, Tc, nsplit, H, V), (uint16_t*)d_hidden + t0 * H,
+                          st);
+    if (rc) return rc;
+  }
+  return ARTK_OK;
+}
+
+size_t artk_grpo_loss_workspace_bytes(int64_t T) {
+  Workspace ws(nullptr, 0);
+  ws.take<float>((size_t)T);
+  ws.take<float>((size_t)T);
+  ws.take<int>(64);
+  return ws.used + 256;
+}
+
+int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const float* advantages,
+                       const uint8_t* mask, const float* weights, const float* ref_logprob,
+                       int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi, float beta,
+                       float* scalars, float* coef, void* workspace, size_t workspace_bytes,
+                       artk_stream_t stream) {
+  ARTK_CHECK_ARG(new_logprob && old_logprob && advantages && mask && weights && scalars,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(T > 0 && S > 0 && T % S == 0, "T must be a positive multiple of S");
+  ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
+  ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
+  Workspace ws(workspace, workspace_bytes);
+  float* pl = ws.take<float>((size_t)T);
+  float* kl = ws.take<float>((size_t)T);
+  int* count = ws.take<int>(64);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, shift, count);
+  ARTK_CHECK_LAUNCH();
+  LossParams p;
+  p.new_lp = new_logprob;
+  p.old_lp = old_logprob;
+  p.adv = advantages;
+  p.mask = mask;
+  p.weights = weights;
+  p.ref_lp = (beta > 0.f) ? ref_logprob : nullptr;
+  p.count = count;
+  p.t0 = 0;
+  p.n = T;
+  p.T = T;
+  p.S = S;
+  p.shift = shift;
+  p.clip_lo = clip_lo;
+  p.clip_hi = clip_hi;
+  p.beta = beta;
+  p.pl_tok = pl;
+  p.kl_tok = kl;
+  p.coef = coef;
+  grpo_loss_tok_kernel<<<(unsigned)((T + 255) / 256), 256, 0, st>>>(p);
+  ARTK_CHECK_LAUNCH();
+  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, p.ref_lp ? beta : 0.f, scalars);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+size_t artk_grpo_fused_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {
+  Workspace ws(nullptr, 0);
+  uint16_t* stash;
+  float2* part;
+  float *sel, *partial, *lse, *coef, *pl, *kl;
+  int nsplit, *count;
+  int64_t Tc = clamp_chunk(T, chunk_tokens);
+  return chunk_workspace(T, V, H, Tc, true, ws, &stash, &part, &sel, &partial, &nsplit, &lse, &coef,
+                         &pl, &kl, &count);
+}
+
+int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_head_t,
+                        const int64_t* tokens, const float* old_logprob, const float* advantages,
+                        const uint8_t* mask, const float* weights, const float* ref_logprob,
+                        int64_t T, int64_t S, int64_t V, int64_t H, float clip_lo, float clip_hi,
+                        float beta, int64_t chunk_tokens, float* scalars, float* logprob,
+                        void* d_hidden, void* workspace, size_t workspace_bytes,
+                        artk_stream_t stream) {
+  int32_t rc = check_common(hidden, lm_head, T, S, V, H, true);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(lm_head_t && tokens && old_logprob && advantages && mask && weights && scalars &&
+                     logprob && d_hidden,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(lm_head_t) && aligned16(d_hidden), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
+  const int64_t Tc = clamp_chunk(T, chunk_tokens);
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* stash;
+  float2* part;
+  float *sel, *partial, *lse, *coef, *pl, *kl;
+  int nsplit, *count;
+  chunk_workspace(T, V, H, Tc, true, ws, &stash, &part, &sel, &partial, &nsplit, &lse, &coef, &pl,
+                  &kl, &count);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const float* ref = (beta > 0.f) ? ref_logprob : nullptr;
+  mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, 1, count);
+  ARTK_CHECK_LAUNCH();
+  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
+    const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
+    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, t0, n, T, S, V, H, part, sel, stash,
+                          logprob + t0, lse + t0, st);
+    if (rc) return rc;
+    LossParams p;
+    p.new_lp = logprob + t0;
+    p.old_lp = old_logprob;
+    p.adv = advantages;
+    p.mask = mask;
+    p.weights = weights;
+    p.ref_lp = ref ? ref + t0 : nullptr;
+    p.count = count;
+    p.t0 = t0;
+    p.n = n;
+    p.T = T;
+    p.S = S;
+    p.shift = 1;
+    p.clip_lo = clip_lo;
+    p.clip_hi = clip_hi;
+    p.beta = beta;
+    p.pl_tok = pl + t0;
+    p.kl_tok = kl + t0;
+    p.coef = coef + t0;
+    grpo_loss_tok_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(p);
+    ARTK_CHECK_LAUNCH();
+    rc = launch_bwd_chunk(stash, lm_head_t, tokens, 1, t0, n, S, V, H, lse + t0, coef + t0, partial,
+                          chunk_nsplit(n, Tc, nsplit, H, V), (uint16_t*)d_hidden + t0 * H, st);
+    if (rc) return rc;
+  }
+  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, ref ? beta : 0.f, scalars);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_transpose_bf16(const void* in, void* out, int64_t R, int64_t C, artk_stream_t stream) {
+  ARTK_CHECK_ARG(in && out, "null pointer argument");
+  ARTK_CHECK_ARG(R > 0 && C > 0, "R and C must be positive");
+  dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64));
+  transpose_bf16_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in, (uint16_t*)out, R,
+                                                               C);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t N, int64_t K,
+                     int32_t out_f32, artk_stream_t stream) {
+  ARTK_CHECK_ARG(P && Q && out, "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(P) && aligned16(Q) && aligned16(out), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(M > 0 && N > 0 && K > 0, "M, N, K must be positive");
+  if (K % BK != 0 || M % 4 != 0) {
+    set_error("K must be a multiple of %d and M a multiple of 4", BK);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  GemmParams p;
+  p.P = P;
+  p.Q = Q;
+  p.out = out;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.MT = (int)((M + TILE - 1) / TILE);
+  p.NT = (int)((N + TILE - 1) / TILE);
+  p.out_f32 = out_f32;
+  gemm_nt_kernel<<<(unsigned)(p.MT * p.NT), NTHREADS, 0, (hipStream_t)stream>>>(p);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+}  // extern "C"

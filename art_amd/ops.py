@@ -1,0 +1,233 @@
+"""Tensor-level wrappers of the artk C-ABI: validate layouts, allocate outputs and
+workspace with torch, pass raw pointers and the current HIP stream.
+
+Every function here requires tensors on a ROCm device and the built HIP
+library; nothing falls back to torch math.
+"""
+from __future__ import annotations
+
+import weakref
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+DEFAULT_CHUNK_TOKENS = 4096
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, name: str, dtype: torch.dtype, shape=None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _mask_u8(mask: torch.Tensor) -> torch.Tensor:
+    if mask.dtype == torch.bool:
+        return mask.view(torch.uint8)
+    if mask.dtype == torch.uint8:
+        return mask
+    raise TypeError(f"mask must be bool or uint8, got {mask.dtype}")
+
+
+# -----------------------------------------------------------------------------
+# transposed copies of frozen weights
+# -----------------------------------------------------------------------------
+_transpose_cache: "dict[int, tuple]" = {}
+
+
+def transpose(x: torch.Tensor) -> torch.Tensor:
+    """out[c, r] = x[r, c] for a contiguous bf16 matrix."""
+    _need(x, "x", torch.bfloat16)
+    if x.dim() != 2:
+        raise ValueError("x must be 2-D")
+    R, C = x.shape
+    out = torch.empty((C, R), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.load().artk_transpose_bf16(x.data_ptr(), out.data_ptr(), R, C, _stream(x.device)))
+    return out
+
+
+def transposed_weight(w: torch.Tensor) -> torch.Tensor:
+    """Transposed copy of a (frozen) weight, cached until the weight is modified
+    in place or freed.  The backward GEMMs need the weight with its other
+    dimension contiguous; the copy is made once per weight version."""
+    key = id(w)
+    hit = _transpose_cache.get(key)
+    if hit is not None:
+        ref, version, ptr, wt = hit
+        if ref() is w and version == w._version and ptr == w.data_ptr():
+            return wt
+    wt = transpose(w)
+    try:
+        ref = weakref.ref(w, lambda _r, k=key: _transpose_cache.pop(k, None))
+    except TypeError:  # pragma: no cover
+        return wt
+    _transpose_cache[key] = (ref, w._version, w.data_ptr(), wt)
+    return wt
+
+
+def gemm_nt(p: torch.Tensor, q: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+    """out[n, m] = sum_k q[n, k] * p[m, k] through the shared MFMA main loop."""
+    _need(p, "p", torch.bfloat16)
+    _need(q, "q", torch.bfloat16)
+    M, K = p.shape
+    N, K2 = q.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    out = torch.empty((N, M), dtype=torch.float32 if out_f32 else torch.bfloat16, device=p.device)
+    _lib.check(
+        _lib.load().artk_gemm_nt(p.data_ptr(), q.data_ptr(), out.data_ptr(), M, N, K, int(out_f32),
+                                 _stream(p.device))
+    )
+    return out
+
+
+# -----------------------------------------------------------------------------
+# logprob forward / backward
+# -----------------------------------------------------------------------------
+def logprob_fwd(hidden: torch.Tensor, lm_head: torch.Tensor, ids: torch.Tensor, shift: bool,
+                row_len: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(logprob, lse), both f32 [T].  hidden bf16 [T,H], lm_head bf16 [V,H], ids int64 [T]."""
+    T, H = hidden.shape
+    V = lm_head.shape[0]
+    _need(hidden, "hidden", torch.bfloat16)
+    _need(lm_head, "lm_head", torch.bfloat16, (V, H))
+    _need(ids, "ids", torch.int64, (T,))
+    lib = _lib.load()
+    dev = hidden.device
+    logprob = torch.empty(T, dtype=torch.float32, device=dev)
+    lse = torch.empty(T, dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_logprob_fwd_workspace_bytes(T, V, H), dev)
+    _lib.check(
+        lib.artk_logprob_fwd(hidden.data_ptr(), lm_head.data_ptr(), ids.data_ptr(), int(shift), T,
+                             row_len, V, H, logprob.data_ptr(), lse.data_ptr(), ws.data_ptr(),
+                             ws.numel(), _stream(dev))
+    )
+    return logprob, lse
+
+
+def logprob_bwd(hidden, lm_head, lm_head_t, ids, shift: bool, row_len: int, lse, grad_logprob,
+                chunk_tokens: int = DEFAULT_CHUNK_TOKENS) -> torch.Tensor:
+    """d_hidden bf16 [T,H] for upstream gradient grad_logprob f32 [T]."""
+    T, H = hidden.shape
+    V = lm_head.shape[0]
+    _need(hidden, "hidden", torch.bfloat16)
+    _need(lm_head, "lm_head", torch.bfloat16, (V, H))
+    _need(lm_head_t, "lm_head_t", torch.bfloat16, (H, V))
+    _need(ids, "ids", torch.int64, (T,))
+    _need(lse, "lse", torch.float32, (T,))
+    _need(grad_logprob, "grad_logprob", torch.float32, (T,))
+    lib = _lib.load()
+    dev = hidden.device
+    d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    ws = _workspace(lib.artk_logprob_bwd_workspace_bytes(T, V, H, chunk_tokens), dev)
+    _lib.check(
+        lib.artk_logprob_bwd(hidden.data_ptr(), lm_head.data_ptr(), lm_head_t.data_ptr(),
+                             ids.data_ptr(), int(shift), T, row_len, V, H, lse.data_ptr(),
+                             grad_logprob.data_ptr(), d_hidden.data_ptr(), chunk_tokens,
+                             ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return d_hidden
+
+
+# -----------------------------------------------------------------------------
+# loss
+# -----------------------------------------------------------------------------
+def clip_bounds(epsilon: float, epsilon_high: Optional[float]) -> Tuple[float, float]:
+    """1 - epsilon and 1 + epsilon_high as the reference forms them in Python
+    floats (src/art/local/train.py:125-131) before torch narrows them to f32."""
+    if epsilon_high is None:
+        epsilon_high = epsilon
+    return 1 - epsilon, 1 + epsilon_high
+
+
+def grpo_loss(new_logprob, old_logprob, advantages, mask, weights, ref_logprob, shift: bool,
+              row_len: int, clip_lo: float, clip_hi: float, beta: float,
+              want_coef: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """scalars f32 [4] = (loss, mean_policy_loss, mean_kl, mask_count) and
+    coef f32 [T] = d loss / d new_logprob."""
+    T = new_logprob.numel()
+    _need(new_logprob, "new_logprob", torch.float32, (T,))
+    _need(old_logprob, "old_logprob", torch.float32, (T,))
+    _need(advantages, "advantages", torch.float32, (T,))
+    _need(weights, "weights", torch.float32, (T,))
+    mask = _need(_mask_u8(mask), "mask", torch.uint8, (T,))
+    if ref_logprob is not None:
+        _need(ref_logprob, "ref_logprob", torch.float32, (T,))
+    lib = _lib.load()
+    dev = new_logprob.device
+    scalars = torch.empty(4, dtype=torch.float32, device=dev)
+    coef = torch.empty(T, dtype=torch.float32, device=dev) if want_coef else None
+    ws = _workspace(lib.artk_grpo_loss_workspace_bytes(T), dev)
+    _lib.check(
+        lib.artk_grpo_loss(new_logprob.data_ptr(), old_logprob.data_ptr(), advantages.data_ptr(),
+                           mask.data_ptr(), weights.data_ptr(), _ptr(ref_logprob), int(shift), T,
+                           row_len, clip_lo, clip_hi, beta, scalars.data_ptr(), _ptr(coef),
+                           ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return scalars, coef
+
+
+def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask, weights,
+               ref_logprob, row_len: int, clip_lo: float, clip_hi: float, beta: float,
+               chunk_tokens: int = DEFAULT_CHUNK_TOKENS, workspace: Optional[torch.Tensor] = None,
+               out: Optional[tuple] = None):
+    """One call for loss and d_hidden of a packed batch given its hidden states.
+
+    All per-token inputs are the un-shifted PackedTensors rows flattened to [T].
+    Returns (scalars f32 [4], logprob f32 [T], d_hidden bf16 [T,H])."""
+    T, H = hidden.shape
+    V = lm_head.shape[0]
+    _need(hidden, "hidden", torch.bfloat16)
+    _need(lm_head, "lm_head", torch.bfloat16, (V, H))
+    _need(lm_head_t, "lm_head_t", torch.bfloat16, (H, V))
+    _need(tokens, "tokens", torch.int64, (T,))
+    _need(old_logprob, "old_logprob", torch.float32, (T,))
+    _need(advantages, "advantages", torch.float32, (T,))
+    _need(weights, "weights", torch.float32, (T,))
+    mask = _need(_mask_u8(mask), "mask", torch.uint8, (T,))
+    if ref_logprob is not None:
+        _need(ref_logprob, "ref_logprob", torch.float32, (T,))
+    lib = _lib.load()
+    dev = hidden.device
+    if out is None:
+        scalars = torch.empty(4, dtype=torch.float32, device=dev)
+        logprob = torch.empty(T, dtype=torch.float32, device=dev)
+        d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    else:
+        scalars, logprob, d_hidden = out
+    need = lib.artk_grpo_fused_workspace_bytes(T, V, H, chunk_tokens)
+    ws = workspace if workspace is not None else _workspace(need, dev)
+    _lib.check(
+        lib.artk_grpo_fused(hidden.data_ptr(), lm_head.data_ptr(), lm_head_t.data_ptr(),
+                            tokens.data_ptr(), old_logprob.data_ptr(), advantages.data_ptr(),
+                            mask.data_ptr(), weights.data_ptr(), _ptr(ref_logprob), T, row_len, V,
+                            H, clip_lo, clip_hi, beta, chunk_tokens, scalars.data_ptr(),
+                            logprob.data_ptr(), d_hidden.data_ptr(), ws.data_ptr(), ws.numel(),
+                            _stream(dev))
+    )
+    return scalars, logprob, d_hidden
+
+
+def grpo_fused_workspace_bytes(T: int, V: int, H: int, chunk_tokens: int = DEFAULT_CHUNK_TOKENS) -> int:
+    return int(_lib.load().artk_grpo_fused_workspace_bytes(T, V, H, chunk_tokens))

@@ -1,0 +1,134 @@
+/*
+ * artk — C-ABI of the MI355X (gfx950) GRPO training hot path.
+ *
+ * Every entry point takes plain device pointers and sizes.  The caller owns all
+ * memory (inputs, outputs and the workspace); the library holds no device
+ * memory, launches on the stream it is given and never synchronises.
+ *
+ * Return value: 0 = ok, negative = argument error (ARTK_ERR_*), positive = the
+ * hipError_t of a failed runtime call.  artk_last_error() returns a
+ * thread-local message for the last non-zero return on the calling thread.
+ *
+ * Layouts: all matrices row-major and contiguous; bf16 = 16-bit brain float;
+ * token ids int64; masks one byte per token (0 / 1); 16-byte aligned pointers.
+ *
+ * "shift": the reference scores position t against token t+1 by shifting every
+ * per-token input one to the left with a pad value
+ * (reference: src/art/local/train.py:284-285, used at :79 and :112-117).
+ * With shift=1 the kernels read element t+1 of the un-shifted [B,S] input (pad
+ * value at the last position of each row) instead of materialising shifted
+ * copies; with shift=0 they read element t.
+ */
+#ifndef ARTK_H_
+#define ARTK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARTK_OK 0
+#define ARTK_ERR_INVALID_ARGUMENT (-1)
+#define ARTK_ERR_WORKSPACE_TOO_SMALL (-2)
+#define ARTK_ERR_UNSUPPORTED_SHAPE (-3)
+
+typedef void* artk_stream_t; /* hipStream_t */
+
+/* Library identification: ABI version (bumped on incompatible change). */
+int32_t artk_abi_version(void);
+const char* artk_last_error(void);
+
+/* ------------------------------------------------------------------------- *
+ * A2 — per-token logprob of the sampled token, forward only.
+ * Replaces: src/art/local/train.py:245-281 (_calculate_logprobs: chunked
+ *   matmul -> gather -> logsumexp -> subtract).  No [T,V] logits are written.
+ *   hidden   bf16 [T,H]      (T = B*S positions)
+ *   lm_head  bf16 [V,H]      (physical layout of the weight whose .t() the
+ *                             reference passes, train.py:76-78)
+ *   ids      int64 [T]       sampled token ids (see "shift"; pad id 0)
+ *   logprob  f32 [T]  out    selected logit - logsumexp
+ *   lse      f32 [T]  out    logsumexp (kept for the backward)
+ * Requires H % 64 == 0, V % 8 == 0.  Ids outside [0,V) give NaN.
+ * ------------------------------------------------------------------------- */
+size_t artk_logprob_fwd_workspace_bytes(int64_t T, int64_t V, int64_t H);
+int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t* ids, int32_t shift,
+                         int64_t T, int64_t S, int64_t V, int64_t H, float* logprob, float* lse,
+                         void* workspace, size_t workspace_bytes, artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * A7 (logprob part) — d_hidden[t,:] = g[t] * (W[y_t,:] - softmax(logits_t) W)
+ * Replaces: autograd backward of train.py:265-272 w.r.t. hidden_states
+ *   (lm_head is frozen: it is not a LoRA target, src/art/dev/model.py:54-62).
+ *   lm_head_t  bf16 [H,V]   transposed copy of lm_head (artk_transpose_bf16)
+ *   lse        f32 [T]      from artk_logprob_fwd
+ *   grad_logprob f32 [T]    upstream gradient per position
+ *   d_hidden   bf16 [T,H] out
+ * Logits are recomputed per chunk of `chunk_tokens` positions into a bounded
+ * bf16 scratch inside the workspace.  Requires H % 64 == 0, V % 64 == 0.
+ * ------------------------------------------------------------------------- */
+size_t artk_logprob_bwd_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens);
+int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm_head_t,
+                         const int64_t* ids, int32_t shift, int64_t T, int64_t S, int64_t V,
+                         int64_t H, const float* lse, const float* grad_logprob, void* d_hidden,
+                         int64_t chunk_tokens, void* workspace, size_t workspace_bytes,
+                         artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * A4 — GRPO clipped-surrogate loss on per-token logprobs, value + gradient.
+ * Replaces: src/art/local/train.py:111-151 (shift, NaN-fill of old logprobs,
+ *   ratio, clip, k3 KL, weight*mask, normalisation by mask.sum()+1e-6) and its
+ *   autograd backward w.r.t. new_logprobs.
+ *   new_logprob f32 [T]   (position frame, i.e. already "shifted")
+ *   old_logprob f32 [T]   NaN = missing            (un-shifted if shift=1)
+ *   advantages  f32 [T], weights f32 [T], mask u8 [T]   (same frame as old)
+ *   ref_logprob f32 [T] or NULL (position frame; used when beta > 0)
+ *   clip_lo / clip_hi     1-epsilon, 1+epsilon_high
+ *   scalars f32 [4] out   {loss, mean_policy_loss, mean_kl, mask_count}
+ *   coef    f32 [T] out   d loss / d new_logprob[t]   (may be NULL)
+ * ------------------------------------------------------------------------- */
+size_t artk_grpo_loss_workspace_bytes(int64_t T);
+int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const float* advantages,
+                       const uint8_t* mask, const float* weights, const float* ref_logprob,
+                       int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi, float beta,
+                       float* scalars, float* coef, void* workspace, size_t workspace_bytes,
+                       artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * A1+A2+A4+A7 fused — loss and d_hidden of one packed batch in one call.
+ * Replaces: the body of compute_loss, src/art/local/train.py:76-151, plus the
+ *   backward that HF Trainer.training_step triggers on its result.
+ * Per chunk of `chunk_tokens` positions: lm_head GEMM with online log-sum-exp
+ * and target gather (bf16 logits of the chunk go to a bounded scratch), loss
+ * coefficients, softmax-gradient in place, d_hidden GEMM against lm_head_t.
+ *   tokens int64 [T], old_logprob/advantages/weights f32 [T], mask u8 [T]:
+ *     the un-shifted PackedTensors rows (src/art/local/pack.py:13-21);
+ *     the shift of train.py:79,112-117 is applied by index arithmetic.
+ *   ref_logprob f32 [T] or NULL   (position frame)
+ *   scalars f32 [4] out, logprob f32 [T] out, d_hidden bf16 [T,H] out
+ * Requires H % 64 == 0, V % 64 == 0.
+ * ------------------------------------------------------------------------- */
+size_t artk_grpo_fused_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens);
+int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_head_t,
+                        const int64_t* tokens, const float* old_logprob, const float* advantages,
+                        const uint8_t* mask, const float* weights, const float* ref_logprob,
+                        int64_t T, int64_t S, int64_t V, int64_t H, float clip_lo, float clip_hi,
+                        float beta, int64_t chunk_tokens, float* scalars, float* logprob,
+                        void* d_hidden, void* workspace, size_t workspace_bytes,
+                        artk_stream_t stream);
+
+/* out[c,r] = in[r,c] for a bf16 [R,C] matrix (R, C multiples of 8).  Used once
+ * per frozen weight to build the K-contiguous operand of the backward GEMMs. */
+int32_t artk_transpose_bf16(const void* in, void* out, int64_t R, int64_t C, artk_stream_t stream);
+
+/* Plain NT GEMM out[n,m] (bf16 or f32) = sum_k Q[n,k] * P[m,k]; exposed for
+ * tests and roofline measurement of the shared main loop.
+ * K % 64 == 0, M % 4 == 0. out_f32: 0 -> bf16 output, 1 -> f32 output. */
+int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t N, int64_t K,
+                     int32_t out_f32, artk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARTK_H_ */
