@@ -41,6 +41,8 @@ SIGNATURES = {
     ),
     "artk_transpose_bf16": (_i32, [_p, _p, _i64, _i64, _p]),
     "artk_gemm_nt": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "artk_profile_enable": (_i32, [_i32]),
+    "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
 }
 
 _lib = None

@@ -59,6 +59,14 @@ struct Workspace {
   bool ok() const { return base != nullptr && used <= size; }
 };
 
+// ---- optional per-kernel timing with HIP events on the launch stream ---------
+// Off by default. When on, the launch helpers bracket each dominant kernel with
+// two events; artk_profile_collect() (after the caller synchronised) sums them.
+enum ProfKind { PROF_LMHEAD_FWD = 0, PROF_DHIDDEN_GEMM = 1, PROF_SOFTMAX_GRAD = 2,
+                PROF_LORA_GEMM = 3, PROF_MOE_GEMM = 4, PROF_KINDS = 8 };
+void prof_begin(int kind, hipStream_t st);
+void prof_end(int kind, hipStream_t st);
+
 // ---- device helpers ---------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -546,10 +546,12 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   fill_f32_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(sel, Tc, NAN);
   ARTK_CHECK_LAUNCH();
   const unsigned grid = (unsigned)(p.VT * p.TT);
+  prof_begin(PROF_LMHEAD_FWD, st);
   if (stash)
     lmhead_fwd_kernel<true><<<grid, NTHREADS, 0, st>>>(p);
   else
     lmhead_fwd_kernel<false><<<grid, NTHREADS, 0, st>>>(p);
+  prof_end(PROF_LMHEAD_FWD, st);
   ARTK_CHECK_LAUNCH();
   lse_finalize_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
                                                                     logprob_chunk, lse_chunk);
@@ -562,8 +564,10 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
                                 int shift, int64_t t0, int64_t Tc, int64_t S, int64_t V, int64_t H,
                                 const float* lse_chunk, const float* coef_chunk, float* partial,
                                 int nsplit, uint16_t* d_hidden_chunk, hipStream_t st) {
+  prof_begin(PROF_SOFTMAX_GRAD, st);
   softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, t0, S,
                                                     shift);
+  prof_end(PROF_SOFTMAX_GRAD, st);
   ARTK_CHECK_LAUNCH();
   BwdParams b;
   b.Wt = lm_head_t;
@@ -576,7 +580,9 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   b.TT = (int)((Tc + TILE - 1) / TILE);
   b.partial = partial;
   b.out = d_hidden_chunk;
+  prof_begin(PROF_DHIDDEN_GEMM, st);
   dhidden_gemm_kernel<<<(unsigned)(b.HT * b.TT * nsplit), NTHREADS, 0, st>>>(b);
+  prof_end(PROF_DHIDDEN_GEMM, st);
   ARTK_CHECK_LAUNCH();
   if (nsplit > 1) {
     const int64_t n4 = Tc * H / 4;

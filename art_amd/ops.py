@@ -231,3 +231,22 @@ def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask
 
 def grpo_fused_workspace_bytes(T: int, V: int, H: int, chunk_tokens: int = DEFAULT_CHUNK_TOKENS) -> int:
     return int(_lib.load().artk_grpo_fused_workspace_bytes(T, V, H, chunk_tokens))
+
+
+# -----------------------------------------------------------------------------
+# per-kernel timing
+# -----------------------------------------------------------------------------
+PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM = range(5)
+
+
+def profile_enable(on: bool) -> None:
+    _lib.check(_lib.load().artk_profile_enable(int(on)))
+
+
+def profile_collect(kind: int) -> Tuple[float, int]:
+    """(summed milliseconds, launches) of one kernel kind; synchronise first."""
+    import ctypes as C
+
+    ms, n = C.c_double(0.0), C.c_int64(0)
+    _lib.check(_lib.load().artk_profile_collect(kind, C.byref(ms), C.byref(n)))
+    return ms.value, n.value

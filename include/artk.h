@@ -128,6 +128,21 @@ int32_t artk_transpose_bf16(const void* in, void* out, int64_t R, int64_t C, art
 int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t N, int64_t K,
                      int32_t out_f32, artk_stream_t stream);
 
+/* ------------------------------------------------------------------------- *
+ * Per-kernel timing (measurement aid; no counterpart in the reference).
+ * artk_profile_enable(1) makes later calls bracket each dominant kernel with
+ * HIP events on the launch stream; after the caller has synchronised,
+ * artk_profile_collect(kind, ...) returns the summed duration and the launch
+ * count of that kind; artk_profile_enable(0) frees the events and turns it off.
+ * ------------------------------------------------------------------------- */
+#define ARTK_PROF_LMHEAD_FWD 0
+#define ARTK_PROF_DHIDDEN_GEMM 1
+#define ARTK_PROF_SOFTMAX_GRAD 2
+#define ARTK_PROF_LORA_GEMM 3
+#define ARTK_PROF_MOE_GEMM 4
+int32_t artk_profile_enable(int32_t on);
+int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches);
+
 #ifdef __cplusplus
 }
 #endif
