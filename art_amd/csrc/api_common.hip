@@ -29,7 +29,7 @@ void prof_begin(int kind, hipStream_t st) {
   std::lock_guard<std::mutex> lk(g_prof_mu);
   hipEvent_t e;
   if (hipEventCreate(&e) != hipSuccess) return;
-  hipEventRecord(e, st);
+  (void)hipEventRecord(e, st);
   g_open[kind] = e;
 }
 
@@ -39,7 +39,7 @@ void prof_end(int kind, hipStream_t st) {
   if (g_open[kind] == nullptr) return;
   hipEvent_t e;
   if (hipEventCreate(&e) != hipSuccess) return;
-  hipEventRecord(e, st);
+  (void)hipEventRecord(e, st);
   g_recs.push_back({g_open[kind], e, kind});
   g_open[kind] = nullptr;
 }
@@ -49,8 +49,8 @@ extern "C" {
 int32_t artk_profile_enable(int32_t on) {
   std::lock_guard<std::mutex> lk(artk::g_prof_mu);
   for (auto& r : artk::g_recs) {
-    hipEventDestroy(r.a);
-    hipEventDestroy(r.b);
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
   }
   artk::g_recs.clear();
   for (auto& e : artk::g_open) e = nullptr;

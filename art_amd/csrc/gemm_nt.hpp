@@ -63,11 +63,12 @@ struct OperandLoader {
     }
   }
 
-  // Issue this wave's 8 DMA instructions for K offset k0 (elements) into the
-  // 32 KiB operand stage at `stage` (LDS byte address, wave-uniform).
+  // Issue DMA instructions LO..HI-1 of this wave's 8 for K offset k0 (elements)
+  // into the 32 KiB operand stage at `stage` (LDS byte address, wave-uniform).
+  template <int LO, int HI>
   __device__ __forceinline__ void issue(char* stage, int wave, int k0) const {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = LO; i < HI; ++i) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * 8 + i) * 1024), 16,
                                                voff[i], k0 * 2, 0, 0);
     }
@@ -120,12 +121,15 @@ __device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
 // of LDS, 1 KiB aligned.
 //
 // Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 16 MFMAs each):
-//   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read
+//   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read;
+//                the second half of the DMA for the next stage is issued here
 //   wait for own LDS reads and own DMA, barrier:
 //                every wave holds its step-3 fragments in registers, so the
 //                current stage is free, and the next stage has landed
-//   DMA for the stage after next goes into the freed buffer
-//   step 3     : MFMAs while step 0 of the next stage is read
+//   step 3     : MFMAs while step 0 of the next stage is read; the first half
+//                of the DMA for the stage after next goes into the freed buffer
+// (the DMA issue is spread over 1.5 steps because the address FIFO of the
+// texture unit backs up and stalls the wave when 16 loads are issued at once)
 // The loop body has no branches: past the end, the DMA re-fetches the last
 // stage into the idle buffer and the fragment prefetch reads values nobody uses.
 __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const void* P, int64_t ldp,
@@ -155,14 +159,15 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
   const int nk = (k_end - k_begin) / BK;
   const int k_last = k_end - BK;
 
-  lp.issue(smem, wave, k_begin);
-  lq.issue(smem + OPER_STAGE_BYTES, wave, k_begin);
+  constexpr int EARLY = 4;  // DMA instructions per operand issued right after the barrier
+  lp.issue<0, 8>(smem, wave, k_begin);
+  lq.issue<0, 8>(smem + OPER_STAGE_BYTES, wave, k_begin);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   {
     int k1 = k_begin + BK < k_last ? k_begin + BK : k_last;
-    lp.issue(smem + STAGE_BYTES, wave, k1);
-    lq.issue(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
+    lp.issue<0, EARLY>(smem + STAGE_BYTES, wave, k1);
+    lq.issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
   }
   Frags f0, f1;
   load_frags(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
@@ -173,6 +178,12 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
     const char* sp = cur + p_wave_off;
     const char* sq = cur + q_wave_off;
 
+    {
+      int k1 = k_begin + (kt + 1) * BK;
+      k1 = k1 < k_last ? k1 : k_last;
+      lp.issue<EARLY, 8>(nxt, wave, k1);
+      lq.issue<EARLY, 8>(nxt + OPER_STAGE_BYTES, wave, k1);
+    }
     load_frags(f1, sp, sq, off[1]);
     mma_frags(acc, f0);
     load_frags(f0, sp, sq, off[2]);
@@ -180,7 +191,13 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
     load_frags(f1, sp, sq, off[3]);
     mma_frags(acc, f0);
 #pragma unroll
-    for (int i = 0; i < 24; ++i) {
+    for (int i = 0; i < 2 * (8 - EARLY); ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+    }
+#pragma unroll
+    for (int i = 0; i < 24 - 2 * (8 - EARLY); ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
     }
@@ -190,14 +207,14 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
 
     int k2 = k_begin + (kt + 2) * BK;
     k2 = k2 < k_last ? k2 : k_last;
-    lp.issue(cur, wave, k2);
-    lq.issue(cur + OPER_STAGE_BYTES, wave, k2);
+    lp.issue<0, EARLY>(cur, wave, k2);
+    lq.issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
     load_frags(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
     mma_frags(acc, f1);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // 2 DMA issues
+      if (i < EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // 2 DMA issues
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
     }
   }
@@ -214,6 +231,22 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
   int x = bid & 7, loc = bid >> 3;
   int start = x * full + (x < rem ? x : rem);
   return start + loc;
+}
+
+
+// Logical tile id -> (row-operand tile, column-operand tile).  Ids walk down a
+// group of GROUP row-operand tiles before moving to the next column-operand
+// tile, so the 32 work-groups that run together on one XCD cover a GROUP x
+// (32/GROUP) patch and share operand panels in that XCD's L2.
+constexpr int TILE_GROUP = 8;
+__device__ __forceinline__ void tile_coords(int id, int row_tiles, int col_tiles, int& rt, int& ct) {
+  const int per = TILE_GROUP * col_tiles;
+  const int g = id / per;
+  const int first = g * TILE_GROUP;
+  const int gs = row_tiles - first < TILE_GROUP ? row_tiles - first : TILE_GROUP;
+  const int w = id - g * per;
+  rt = first + w % gs;
+  ct = w / gs;
 }
 
 }  // namespace artk

@@ -55,7 +55,8 @@ template <bool STASH>
 __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
-  const int vt = id / p.TT, tt = id % p.TT;
+  int vt, tt;
+  tile_coords(id, p.VT, p.TT, vt, tt);
 
   TileAcc acc;
   acc.zero();
@@ -149,24 +150,43 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
   }
 }
 
-// K2: merge the per-tile (max, sumexp) partials of each position.
+// K2: merge the per-tile (max, sumexp) partials of each position.  A block
+// handles 16 positions; 16 threads per position each merge a strided share of
+// the partials online, then the 16 shares are merged through LDS.
 __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restrict__ part,
                                                            int nparts, int64_t Tc,
                                                            const float* __restrict__ sel,
                                                            float* __restrict__ logprob,
                                                            float* __restrict__ lse) {
-  int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= Tc) return;
-  float M = -INFINITY;
-  for (int i = 0; i < nparts; ++i) M = fmaxf(M, part[(int64_t)i * Tc + t].x);
-  float L = 0.f;
-  for (int i = 0; i < nparts; ++i) {
-    float2 v = part[(int64_t)i * Tc + t];
-    L += v.y * __builtin_amdgcn_exp2f((v.x - M) * LOG2E);
+  __shared__ float2 red[16][17];
+  const int tl = threadIdx.x & 15, sl = threadIdx.x >> 4;
+  const int64_t t = (int64_t)blockIdx.x * 16 + tl;
+  float m = -INFINITY, l = 0.f;
+  if (t < Tc) {
+    for (int i = sl; i < nparts; i += 16) {
+      const float2 v = part[(int64_t)i * Tc + t];
+      const float mn = fmaxf(m, v.x);
+      if (mn != -INFINITY)
+        l = l * __builtin_amdgcn_exp2f((m - mn) * LOG2E) + v.y * __builtin_amdgcn_exp2f((v.x - mn) * LOG2E);
+      m = mn;
+    }
   }
-  float z = M + logf(L);
-  lse[t] = z;
-  logprob[t] = sel[t] - z;
+  red[sl][tl] = make_float2(m, l);
+  __syncthreads();
+  if (sl == 0 && t < Tc) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) M = fmaxf(M, red[i][tl].x);
+    float L = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float2 v = red[i][tl];
+      if (v.x != -INFINITY) L += v.y * __builtin_amdgcn_exp2f((v.x - M) * LOG2E);
+    }
+    const float z = M + logf(L);
+    lse[t] = z;
+    logprob[t] = sel[t] - z;
+  }
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -344,7 +364,8 @@ __global__ __launch_bounds__(NTHREADS) void dhidden_gemm_kernel(BwdParams p) {
   const int tiles = p.HT * p.TT;
   const int split = id / tiles;
   const int rem = id - split * tiles;
-  const int ht = rem / p.TT, tt = rem % p.TT;
+  int ht, tt;
+  tile_coords(rem, p.HT, p.TT, ht, tt);
   const int KT = (int)(p.V / BK);
   const int kb = (int)((int64_t)split * KT / p.nsplit);
   const int ke = (int)((int64_t)(split + 1) * KT / p.nsplit);
@@ -431,7 +452,8 @@ struct GemmParams {
 __global__ __launch_bounds__(NTHREADS) void gemm_nt_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
-  const int mt = id / p.NT, nt = id % p.NT;
+  int mt, nt;
+  tile_coords(id, p.MT, p.NT, mt, nt);
   TileAcc acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
@@ -553,7 +575,7 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
     lmhead_fwd_kernel<false><<<grid, NTHREADS, 0, st>>>(p);
   prof_end(PROF_LMHEAD_FWD, st);
   ARTK_CHECK_LAUNCH();
-  lse_finalize_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
+  lse_finalize_kernel<<<(unsigned)((Tc + 15) / 16), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
                                                                     logprob_chunk, lse_chunk);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
