@@ -41,6 +41,12 @@ SIGNATURES = {
     ),
     "artk_transpose_bf16": (_i32, [_p, _p, _i64, _i64, _p]),
     "artk_gemm_nt": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
+    "artk_lora_linear_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "artk_lora_linear_fwd": (
+        _i32, [_p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
+    "artk_lora_linear_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "artk_lora_linear_bwd": (
+        _i32, [_p, _p, _p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),
     "artk_profile_enable": (_i32, [_i32]),
     "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
 }

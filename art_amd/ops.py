@@ -234,6 +234,54 @@ def grpo_fused_workspace_bytes(T: int, V: int, H: int, chunk_tokens: int = DEFAU
 
 
 # -----------------------------------------------------------------------------
+# LoRA linear
+# -----------------------------------------------------------------------------
+def lora_linear_fwd(x, W, A, B, scale: float):
+    """(y bf16 [T,out], xa f32 [T,r]) for x bf16 [T,in], W bf16 [out,in], A bf16 [r,in], B bf16 [out,r]."""
+    T, n_in = x.shape
+    n_out, r = B.shape
+    _need(x, "x", torch.bfloat16)
+    _need(W, "W", torch.bfloat16, (n_out, n_in))
+    _need(A, "A", torch.bfloat16, (r, n_in))
+    _need(B, "B", torch.bfloat16, (n_out, r))
+    lib = _lib.load()
+    dev = x.device
+    y = torch.empty((T, n_out), dtype=torch.bfloat16, device=dev)
+    xa = torch.empty((T, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_lora_linear_fwd_workspace_bytes(T, n_in, n_out, r), dev)
+    _lib.check(
+        lib.artk_lora_linear_fwd(x.data_ptr(), W.data_ptr(), A.data_ptr(), B.data_ptr(), scale, T,
+                                 n_in, n_out, r, y.data_ptr(), xa.data_ptr(), ws.data_ptr(),
+                                 ws.numel(), _stream(dev))
+    )
+    return y, xa
+
+
+def lora_linear_bwd(g, x, W_t, A, B, xa, scale: float):
+    """(dx bf16 [T,in], dA f32 [r,in], dB f32 [out,r]) for upstream gradient g bf16 [T,out]."""
+    T, n_in = x.shape
+    n_out, r = B.shape
+    _need(g, "g", torch.bfloat16, (T, n_out))
+    _need(x, "x", torch.bfloat16)
+    _need(W_t, "W_t", torch.bfloat16, (n_in, n_out))
+    _need(A, "A", torch.bfloat16, (r, n_in))
+    _need(B, "B", torch.bfloat16, (n_out, r))
+    _need(xa, "xa", torch.float32, (T, r))
+    lib = _lib.load()
+    dev = x.device
+    dx = torch.empty((T, n_in), dtype=torch.bfloat16, device=dev)
+    dA = torch.empty((r, n_in), dtype=torch.float32, device=dev)
+    dB = torch.empty((n_out, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_lora_linear_bwd_workspace_bytes(T, n_in, n_out, r), dev)
+    _lib.check(
+        lib.artk_lora_linear_bwd(g.data_ptr(), x.data_ptr(), W_t.data_ptr(), A.data_ptr(),
+                                 B.data_ptr(), xa.data_ptr(), scale, T, n_in, n_out, r, dx.data_ptr(),
+                                 dA.data_ptr(), dB.data_ptr(), ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return dx, dA, dB
+
+
+# -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------
 PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM = range(5)

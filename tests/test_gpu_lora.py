@@ -1,0 +1,101 @@
+"""GPU parity of the LoRA linear (forward and backward) against the CPU oracle.
+
+Tolerance: rel-L2 <= 1e-2 for y, dx, dA, dB against the fp32 oracle evaluated
+on the same bf16-valued inputs."""
+import math
+import os
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+import lora_oracle  # noqa: E402
+
+from art_amd import ops  # noqa: E402
+from art_amd.lora import LoRALinear, lora_linear  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def rel_l2(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+
+def make(T, n_in, n_out, r, seed, b_std=0.01):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, n_in, generator=g).to(torch.bfloat16)
+    W = (0.02 * torch.randn(n_out, n_in, generator=g)).to(torch.bfloat16)
+    bound = 1.0 / math.sqrt(n_in)  # Kaiming-uniform with a = sqrt(5)
+    A = ((torch.rand(r, n_in, generator=g) * 2 - 1) * bound).to(torch.bfloat16)
+    B = (b_std * torch.randn(n_out, r, generator=g)).to(torch.bfloat16)
+    up = torch.randn(T, n_out, generator=g).to(torch.bfloat16)
+    return x, W, A, B, up
+
+
+def run_gpu(x, W, A, B, up, scale, gpu):
+    xd, Wd, Ad, Bd, upd = (t.to(gpu) for t in (x, W, A, B, up))
+    y, xa = ops.lora_linear_fwd(xd, Wd, Ad, Bd, scale)
+    dx, dA, dB = ops.lora_linear_bwd(upd, xd, ops.transpose(Wd), Ad, Bd, xa, scale)
+    return y.cpu().float(), dx.cpu().float(), dA.cpu(), dB.cpu()
+
+
+@pytest.mark.parametrize("T,n_in,n_out,r", [(512, 256, 256, 8), (300, 192, 320, 8), (256, 128, 64, 16),
+                                            (1000, 512, 576, 24)])
+def test_lora_matches_oracle(artk_lib, gpu, T, n_in, n_out, r):
+    print(f"lora T={T} in={n_in} out={n_out} r={r}", flush=True)
+    x, W, A, B, up = make(T, n_in, n_out, r, T + r)
+    scale = 16 / r
+    y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, scale, up)
+    y, dx, dA, dB = run_gpu(x, W, A, B, up, scale, gpu)
+    assert rel_l2(y, y0) <= TOL
+    assert rel_l2(dx, dx0) <= TOL
+    assert rel_l2(dA, dA0) <= TOL
+    assert rel_l2(dB, dB0) <= TOL
+
+
+def test_lora_zero_factors(artk_lib, gpu):
+    """B = 0: y is the base projection and dA vanishes; A = 0: dB vanishes."""
+    x, W, A, B, up = make(256, 128, 192, 8, 5)
+    y, dx, dA, dB = run_gpu(x, W, A, torch.zeros_like(B), up, 2.0, gpu)
+    base = ops.gemm_nt(W.to(gpu), x.to(gpu)).cpu().float()
+    assert torch.equal(y, base)
+    assert dA.abs().max().item() == 0.0
+    assert dB.abs().max().item() > 0.0
+    y, dx, dA, dB = run_gpu(x, W, torch.zeros_like(A), B, up, 2.0, gpu)
+    assert dB.abs().max().item() == 0.0
+    assert dA.abs().max().item() > 0.0
+
+
+@pytest.mark.parametrize("n_out", [2048, 256, 11008])
+def test_lora_config2_full_size(artk_lib, gpu, n_out):
+    """BASELINE config 2 (Qwen2.5-3B projections) at full size."""
+    print(f"lora config2 out={n_out}", flush=True)
+    x, W, A, B, up = make(8192, 2048, n_out, 8, 1002 + n_out)
+    y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, 2.0, up)
+    y, dx, dA, dB = run_gpu(x, W, A, B, up, 2.0, gpu)
+    assert rel_l2(y, y0) <= TOL
+    assert rel_l2(dx, dx0) <= TOL
+    assert rel_l2(dA, dA0) <= TOL
+    assert rel_l2(dB, dB0) <= TOL
+
+
+def test_lora_module_autograd(artk_lib, gpu):
+    torch.manual_seed(0)
+    mod = LoRALinear(256, 320, r=8, lora_alpha=16, device=gpu, dtype=torch.float32)
+    with torch.no_grad():
+        mod.lora_B.normal_(std=0.01)
+    x = torch.randn(2, 96, 256, device=gpu, dtype=torch.bfloat16, requires_grad=True)
+    y = mod(x)
+    assert y.shape == (2, 96, 320)
+    up = torch.randn_like(y)
+    y.backward(up)
+    y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(
+        x.detach().cpu().view(-1, 256), mod.weight.cpu(), mod.lora_A.detach().cpu().to(torch.bfloat16),
+        mod.lora_B.detach().cpu().to(torch.bfloat16), mod.scaling, up.cpu().view(-1, 320))
+    assert rel_l2(y.detach().cpu().float().view(-1, 320), y0) <= TOL
+    assert rel_l2(x.grad.cpu().float().view(-1, 256), dx0) <= TOL
+    assert rel_l2(mod.lora_A.grad.cpu(), dA0) <= TOL
+    assert rel_l2(mod.lora_B.grad.cpu(), dB0) <= TOL
+    assert mod.weight.grad is None
