@@ -47,9 +47,12 @@ struct OperandLoader {
   // base: first element of the operand; ld: leading dimension in elements;
   // row0: first tile row; nrows: rows the operand really has (rows past the
   // end are clamped to the last valid row; the epilogue never stores them).
+  // gather (optional): tile row i reads operand row gather[row0 + i] instead of
+  // row0 + i; all gathered rows must lie within 2 GiB of `base`.
   __device__ __forceinline__ void init(const void* base, int64_t ld, int64_t row0,
-                                       int64_t nrows, int wave, int lane) {
-    const char* p = (const char*)base + row0 * ld * 2;
+                                       int64_t nrows, int wave, int lane,
+                                       const int* gather = nullptr) {
+    const char* p = (const char*)base + (gather ? 0 : row0 * ld * 2);
     rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
     int64_t left = nrows - row0;
     int nvalid = left >= TILE ? TILE : (int)left;
@@ -58,7 +61,8 @@ struct OperandLoader {
     for (int i = 0; i < 8; ++i) {
       int row = (wave * 8 + i) * 8 + r;
       int kc = pc ^ swz(row);
-      int rc = row < nvalid ? row : nvalid - 1;
+      int64_t rc = row < nvalid ? row : nvalid - 1;
+      if (gather) rc = gather[row0 + rc];
       voff[i] = (int)(rc * ld * 2) + kc * 16;
     }
   }
@@ -135,7 +139,7 @@ __device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
 __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const void* P, int64_t ldp,
                                              int64_t prow0, int64_t prows, const void* Q,
                                              int64_t ldq, int64_t qrow0, int64_t qrows, int k_begin,
-                                             int k_end) {
+                                             int k_end, const int* qgather = nullptr) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -143,7 +147,7 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
 
   OperandLoader lp, lq;
   lp.init(P, ldp, prow0, prows, wave, lane);
-  lq.init(Q, ldq, qrow0, qrows, wave, lane);
+  lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather);
 
   // Per-lane LDS read offsets (within an operand stage) for the 4 K=16 steps.
   int off[4];

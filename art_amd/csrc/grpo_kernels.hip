@@ -308,24 +308,94 @@ __global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __r
 }
 
 // ----------------------------------------------------------------------------
-// K3: in-place softmax gradient on the bf16 logits scratch:
+// K3a: active rows of a chunk (coef != 0) in ascending order, the inverse map,
+// and the schedule of the d_hidden GEMM over those rows.  One block.
+//   sched[0] = n_active, [1] = token tiles, [2] = K splits, [3] = work-groups
+// Rows whose coefficient is zero (non-assistant positions, zero advantage) have
+// an exactly zero d_hidden row and are skipped by K3b and K4.
+__global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restrict__ coef, int Tc,
+                                                            int HT, int ksteps, int part_rows,
+                                                            int num_cus, int* __restrict__ active_idx,
+                                                            int* __restrict__ pos,
+                                                            int* __restrict__ sched) {
+  __shared__ int wave_tot[16];
+  __shared__ int total;
+  const int per = (Tc + 1023) / 1024;
+  const int r0 = threadIdx.x * per;
+  int cnt = 0;
+  for (int i = 0; i < per; ++i) {
+    int r = r0 + i;
+    if (r < Tc && coef[r] != 0.f) ++cnt;
+  }
+  // exclusive scan of cnt over the block
+  int incl = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int v = __shfl_up(incl, o, 64);
+    if ((threadIdx.x & 63) >= o) incl += v;
+  }
+  if ((threadIdx.x & 63) == 63) wave_tot[threadIdx.x >> 6] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int w = 0; w < 16; ++w) {
+      int v = wave_tot[w];
+      wave_tot[w] = run;
+      run += v;
+    }
+    total = run;
+  }
+  __syncthreads();
+  int at = wave_tot[threadIdx.x >> 6] + incl - cnt;
+  for (int i = 0; i < per; ++i) {
+    int r = r0 + i;
+    if (r >= Tc) break;
+    if (coef[r] != 0.f) {
+      active_idx[at] = r;
+      pos[r] = at;
+      ++at;
+    } else {
+      pos[r] = -1;
+    }
+  }
+  if (threadIdx.x == 0) {
+    const int n = total;
+    const int tta = (n + TILE - 1) / TILE;
+    const int tiles = HT * tta;
+    int best = 1;
+    float best_eff = 0.f;
+    for (int ns = 1; ns <= 16 && tiles > 0; ++ns) {
+      if (ns > 1 && (ksteps / ns < 32 || ns * tta * TILE > part_rows)) break;
+      int blocks = tiles * ns;
+      int rounds = (blocks + num_cus - 1) / num_cus;
+      float eff = (float)blocks / ((float)rounds * num_cus);
+      if (eff > best_eff + 0.02f) {
+        best_eff = eff;
+        best = ns;
+      }
+    }
+    sched[0] = n;
+    sched[1] = tta;
+    sched[2] = best;
+    sched[3] = tiles * best;
+  }
+}
+
+// K3b: in-place softmax gradient on the bf16 logits scratch, active rows only:
 //   P[t,v] = coef[t] * ( [v == y_t] - exp(z[t,v] - lse[t]) )
-// One block per position; rows with coef == 0 are zero-filled without a read.
-// ----------------------------------------------------------------------------
+// One block per active row.
 __global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict__ stash, int64_t V,
                                                            const float* __restrict__ lse,
                                                            const float* __restrict__ coef,
                                                            const int64_t* __restrict__ ids,
-                                                           int64_t t0, int64_t S, int shift) {
-  const int64_t r = blockIdx.x;
+                                                           int64_t t0, int64_t S, int shift,
+                                                           const int* __restrict__ active_idx,
+                                                           const int* __restrict__ sched) {
+  if ((int)blockIdx.x >= sched[0]) return;
+  const int64_t r = active_idx[blockIdx.x];
   uint4* row = (uint4*)(stash + r * V);
   const int nvec = (int)(V >> 3);
   const float c = coef[r];
-  if (c == 0.f) {
-    const uint4 z = make_uint4(0, 0, 0, 0);
-    for (int i = threadIdx.x; i < nvec; i += 256) row[i] = z;
-    return;
-  }
   const int64_t y = target_id(ids, t0 + r, S, shift);
   const float nl = -lse[r] * LOG2E;
   for (int i = threadIdx.x; i < nvec; i += 256) {
@@ -350,70 +420,76 @@ __global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict_
 // K4: d_hidden tile = P[256 positions, k-range of V] x lm_head_t[256 h, same]^T
 // ----------------------------------------------------------------------------
 struct BwdParams {
-  const void* Wt;    // [H,V] bf16
-  const void* P;     // [Tc,V] bf16
-  int64_t V, H, Tc;
-  int nsplit, HT, TT;
-  float* partial;    // [nsplit][Tc][H] when nsplit > 1
-  uint16_t* out;     // [Tc,H] bf16 when nsplit == 1
+  const void* Wt;          // [H,V] bf16
+  const void* P;           // [Tc,V] bf16 (only active rows hold gradients)
+  int64_t V, H;
+  int HT;
+  const int* active_idx;   // [n_active] rows of P, ascending
+  const int* sched;        // see compact_rows_kernel
+  float* partial;          // [nsplit][tiles*256][H] f32
 };
 
+// The grid is sized for the worst case (every row active); the work-groups
+// beyond the device-side schedule exit at once.
 __global__ __launch_bounds__(NTHREADS) void dhidden_gemm_kernel(BwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  const int tiles = p.HT * p.TT;
+  const int n_active = p.sched[0], TT = p.sched[1], nsplit = p.sched[2], n_work = p.sched[3];
+  if ((int)blockIdx.x >= n_work) return;
+  const int id = xcd_remap(blockIdx.x, n_work);
+  const int tiles = p.HT * TT;
   const int split = id / tiles;
   const int rem = id - split * tiles;
   int ht, tt;
-  tile_coords(rem, p.HT, p.TT, ht, tt);
+  tile_coords(rem, p.HT, TT, ht, tt);
   const int KT = (int)(p.V / BK);
-  const int kb = (int)((int64_t)split * KT / p.nsplit);
-  const int ke = (int)((int64_t)(split + 1) * KT / p.nsplit);
+  const int kb = (int)((int64_t)split * KT / nsplit);
+  const int ke = (int)((int64_t)(split + 1) * KT / nsplit);
 
   TileAcc acc;
   acc.zero();
-  gemm_tile_nt(acc, smem, p.Wt, p.V, (int64_t)ht * TILE, p.H, p.P, p.V, (int64_t)tt * TILE, p.Tc,
-               kb * BK, ke * BK);
+  gemm_tile_nt(acc, smem, p.Wt, p.V, (int64_t)ht * TILE, p.H, p.P, p.V, (int64_t)tt * TILE,
+               n_active, kb * BK, ke * BK, p.active_idx);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int half = lane >> 5;
+  const int64_t rows_per_split = (int64_t)TT * TILE;
 #pragma unroll
   for (int ni = 0; ni < 4; ++ni) {
-    const int col = tt * TILE + acc_col(wn, ni, lane);
-    if (col >= p.Tc) continue;
+    const int col = tt * TILE + acc_col(wn, ni, lane);  // compact row
+    if (col >= n_active) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int64_t h = (int64_t)ht * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
         if (h >= p.H) continue;
-        if (p.nsplit == 1) {
-          bf16x4 o;
+        floatx4 o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
-          *(bf16x4*)(p.out + (int64_t)col * p.H + h) = o;
-        } else {
-          floatx4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = acc.c[mi][ni][q * 4 + e];
-          *(floatx4*)(p.partial + ((int64_t)split * p.Tc + col) * p.H + h) = o;
-        }
+        for (int e = 0; e < 4; ++e) o[e] = acc.c[mi][ni][q * 4 + e];
+        *(floatx4*)(p.partial + ((int64_t)split * rows_per_split + col) * p.H + h) = o;
       }
   }
 }
 
-// K5: out = bf16(sum over splits of partial), 4 elements per thread.
+// K5: d_hidden row r = bf16(sum over splits of partial[compact row of r]) or 0
+// for inactive rows; 4 elements per thread.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
-                                                            int nsplit, int64_t n4,
-                                                            uint16_t* __restrict__ out) {
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n4) return;
-  floatx4 s = ((const floatx4*)partial)[i];
-  for (int k = 1; k < nsplit; ++k) {
-    floatx4 v = ((const floatx4*)partial)[(int64_t)k * n4 + i];
-    s += v;
+                                                            const int* __restrict__ pos,
+                                                            const int* __restrict__ sched, int64_t Tc,
+                                                            int64_t H, uint16_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t h4 = H / 4;
+  if (i >= Tc * h4) return;
+  const int64_t r = i / h4, c = i - r * h4;
+  const int pr = pos[r];
+  floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  if (pr >= 0) {
+    const int nsplit = sched[2];
+    const int64_t rows_per_split = (int64_t)sched[1] * TILE;
+    for (int k = 0; k < nsplit; ++k)
+      s += ((const floatx4*)(partial + ((int64_t)k * rows_per_split + pr) * H))[c];
   }
   bf16x4 o;
 #pragma unroll
@@ -581,14 +657,35 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   return ARTK_OK;
 }
 
-// Launch K3, K4 (+K5) for one chunk whose bf16 logits are in `stash`.
+// fp32 partial rows of the d_hidden GEMM for a chunk of Tc rows: enough for the
+// split count the dense case would use.
+static int64_t bwd_part_rows(int64_t Tc, int64_t H, int64_t V) {
+  const int64_t tt = (Tc + TILE - 1) / TILE;
+  const int tiles = (int)(((H + TILE - 1) / TILE) * tt);
+  return (int64_t)choose_nsplit(tiles, (int)(V / BK)) * tt * TILE;
+}
+
+struct BwdScratch {
+  float* partial;
+  int64_t part_rows;
+  int* active_idx;
+  int* pos;
+  int* sched;
+};
+
+// Launch K3a, K3b, K4, K5 for one chunk whose bf16 logits are in `stash`.
 static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const int64_t* ids,
                                 int shift, int64_t t0, int64_t Tc, int64_t S, int64_t V, int64_t H,
-                                const float* lse_chunk, const float* coef_chunk, float* partial,
-                                int nsplit, uint16_t* d_hidden_chunk, hipStream_t st) {
+                                const float* lse_chunk, const float* coef_chunk, const BwdScratch& sc,
+                                uint16_t* d_hidden_chunk, hipStream_t st) {
+  const int HT = (int)((H + TILE - 1) / TILE);
+  const int TT = (int)((Tc + TILE - 1) / TILE);
+  compact_rows_kernel<<<1, 1024, 0, st>>>(coef_chunk, (int)Tc, HT, (int)(V / BK), (int)sc.part_rows,
+                                          num_cus(), sc.active_idx, sc.pos, sc.sched);
+  ARTK_CHECK_LAUNCH();
   prof_begin(PROF_SOFTMAX_GRAD, st);
   softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, t0, S,
-                                                    shift);
+                                                    shift, sc.active_idx, sc.sched);
   prof_end(PROF_SOFTMAX_GRAD, st);
   ARTK_CHECK_LAUNCH();
   BwdParams b;
@@ -596,38 +693,22 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   b.P = stash;
   b.V = V;
   b.H = H;
-  b.Tc = Tc;
-  b.nsplit = nsplit;
-  b.HT = (int)((H + TILE - 1) / TILE);
-  b.TT = (int)((Tc + TILE - 1) / TILE);
-  b.partial = partial;
-  b.out = d_hidden_chunk;
+  b.HT = HT;
+  b.active_idx = sc.active_idx;
+  b.sched = sc.sched;
+  b.partial = sc.partial;
+  const int64_t max_blocks = sc.part_rows / TILE * HT;  // tiles * splits can never exceed this
+  const int64_t dense_cap = (int64_t)HT * TT * 16;
+  const unsigned grid = (unsigned)(max_blocks < dense_cap ? max_blocks : dense_cap);
   prof_begin(PROF_DHIDDEN_GEMM, st);
-  dhidden_gemm_kernel<<<(unsigned)(b.HT * b.TT * nsplit), NTHREADS, 0, st>>>(b);
+  dhidden_gemm_kernel<<<grid, NTHREADS, 0, st>>>(b);
   prof_end(PROF_DHIDDEN_GEMM, st);
   ARTK_CHECK_LAUNCH();
-  if (nsplit > 1) {
-    const int64_t n4 = Tc * H / 4;
-    splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(partial, nsplit, n4,
-                                                                       d_hidden_chunk);
-    ARTK_CHECK_LAUNCH();
-  }
+  const int64_t n4 = Tc * H / 4;
+  splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(sc.partial, sc.pos, sc.sched, Tc,
+                                                                     H, d_hidden_chunk);
+  ARTK_CHECK_LAUNCH();
   return ARTK_OK;
-}
-
-static int bwd_nsplit(int64_t Tc, int64_t H, int64_t V) {
-  int tiles = (int)(((H + TILE - 1) / TILE) * ((Tc + TILE - 1) / TILE));
-  return choose_nsplit(tiles, (int)(V / BK));
-}
-
-// Split count for a chunk of n <= Tc positions that must fit the fp32 partial
-// buffer sized for `nsplit` splits of Tc positions.
-static int chunk_nsplit(int64_t n, int64_t Tc, int nsplit, int64_t H, int64_t V) {
-  if (nsplit <= 1) return 1;
-  if (n == Tc) return nsplit;
-  int ns = bwd_nsplit(n, H, V);
-  while (ns > 1 && (int64_t)ns * n > (int64_t)nsplit * Tc) --ns;
-  return ns;
 }
 
 }  // namespace artk
@@ -664,43 +745,55 @@ int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t*
                           lse, (hipStream_t)stream);
 }
 
-static size_t chunk_workspace(int64_t T, int64_t V, int64_t H, int64_t Tc, bool with_loss,
-                              Workspace& ws, uint16_t** stash, float2** part, float** sel,
-                              float** partial, int* nsplit, float** lse, float** coef, float** pl,
-                              float** kl, int** count) {
-  int64_t VT = (V + TILE - 1) / TILE;
-  *stash = ws.take<uint16_t>((size_t)(Tc * V));
-  *part = ws.take<float2>((size_t)(2 * VT * Tc));
-  *sel = ws.take<float>((size_t)Tc);
-  *nsplit = bwd_nsplit(Tc, H, V);
-  *partial = *nsplit > 1 ? ws.take<float>((size_t)(*nsplit) * Tc * H) : nullptr;
-  if (with_loss) {
-    *lse = ws.take<float>((size_t)T);
-    *coef = ws.take<float>((size_t)T);
-    *pl = ws.take<float>((size_t)T);
-    *kl = ws.take<float>((size_t)T);
-    *count = ws.take<int>(64);
+// Scratch of one chunk of Tc positions carved out of the caller's workspace.
+struct ChunkScratch {
+  uint16_t* stash;  // [Tc,V] bf16 logits, then softmax gradient
+  float2* part;     // [2*VT][Tc]
+  float* sel;       // [Tc]
+  BwdScratch bwd;
+  float *lse, *coef, *pl, *kl;  // [T] each (fused op only)
+  int* count;
+  float *lp_tmp, *lse_tmp;      // [Tc] each (standalone backward only)
+};
+
+static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bool fused,
+                  ChunkScratch& c) {
+  const int64_t VT = (V + TILE - 1) / TILE;
+  c.stash = ws.take<uint16_t>((size_t)(Tc * V));
+  c.part = ws.take<float2>((size_t)(2 * VT * Tc));
+  c.sel = ws.take<float>((size_t)Tc);
+  c.bwd.part_rows = bwd_part_rows(Tc, H, V);
+  c.bwd.partial = ws.take<float>((size_t)c.bwd.part_rows * H);
+  c.bwd.active_idx = ws.take<int>((size_t)Tc);
+  c.bwd.pos = ws.take<int>((size_t)Tc);
+  c.bwd.sched = ws.take<int>(64);
+  if (fused) {
+    c.lse = ws.take<float>((size_t)T);
+    c.coef = ws.take<float>((size_t)T);
+    c.pl = ws.take<float>((size_t)T);
+    c.kl = ws.take<float>((size_t)T);
+    c.count = ws.take<int>(64);
+  } else {
+    c.lp_tmp = ws.take<float>((size_t)Tc);
+    c.lse_tmp = ws.take<float>((size_t)Tc);
   }
-  return ws.used + 256;
 }
 
-static int64_t clamp_chunk(int64_t T, int64_t chunk_tokens) {
+// Chunk length: the caller's wish, at most T, and small enough that a row
+// offset inside the logits scratch fits the 31-bit offsets of the GEMM loader.
+static int64_t clamp_chunk(int64_t T, int64_t V, int64_t chunk_tokens) {
   if (chunk_tokens <= 0) chunk_tokens = 4096;
+  const int64_t cap = ((1ll << 30) - 1) / V / TILE * TILE;  // Tc * V * 2 bytes < 2^31
+  if (chunk_tokens > cap) chunk_tokens = cap > TILE ? cap : TILE;
   if (chunk_tokens > T) chunk_tokens = T;
   return chunk_tokens;
 }
 
 size_t artk_logprob_bwd_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {
   Workspace ws(nullptr, 0);
-  uint16_t* stash;
-  float2* part;
-  float *sel, *partial, *lse, *coef, *pl, *kl;
-  int nsplit, *count;
-  int64_t Tc = clamp_chunk(T, chunk_tokens);
-  size_t n = chunk_workspace(T, V, H, Tc, false, ws, &stash, &part, &sel, &partial, &nsplit, &lse,
-                             &coef, &pl, &kl, &count);
-  // scratch logprob / lse outputs of the recompute pass
-  return n + 2 * align_up((size_t)Tc * 4, 256) + 512;
+  ChunkScratch c;
+  carve(ws, T, V, H, clamp_chunk(T, V, chunk_tokens), false, c);
+  return ws.used + 256;
 }
 
 int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm_head_t,
@@ -713,16 +806,10 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
   ARTK_CHECK_ARG(lm_head_t && ids && lse && grad_logprob && d_hidden, "null pointer argument");
   ARTK_CHECK_ARG(aligned16(lm_head_t) && aligned16(d_hidden), "pointers must be 16-byte aligned");
   ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
-  const int64_t Tc = clamp_chunk(T, chunk_tokens);
+  const int64_t Tc = clamp_chunk(T, V, chunk_tokens);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* stash;
-  float2* part;
-  float *sel, *partial, *lse_u, *coef_u, *pl_u, *kl_u;
-  int nsplit, *count_u;
-  chunk_workspace(T, V, H, Tc, false, ws, &stash, &part, &sel, &partial, &nsplit, &lse_u, &coef_u,
-                  &pl_u, &kl_u, &count_u);
-  float* lp_tmp = ws.take<float>((size_t)Tc);
-  float* lse_tmp = ws.take<float>((size_t)Tc);
+  ChunkScratch c;
+  carve(ws, T, V, H, Tc, false, c);
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
@@ -730,13 +817,12 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
   hipStream_t st = (hipStream_t)stream;
   for (int64_t t0 = 0; t0 < T; t0 += Tc) {
     const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
-    // The stash row pitch is V, so a shorter last chunk simply uses fewer rows.
-    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, t0, n, T, S, V, H, part, sel, stash, lp_tmp,
-                          lse_tmp, st);
+    // The scratch row pitch is V, so a shorter last chunk simply uses fewer rows.
+    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, t0, n, T, S, V, H, c.part, c.sel, c.stash,
+                          c.lp_tmp, c.lse_tmp, st);
     if (rc) return rc;
-    rc = launch_bwd_chunk(stash, lm_head_t, ids, shift, t0, n, S, V, H, lse + t0, grad_logprob + t0,
-                          partial, chunk_nsplit(n, Tc, nsplit, H, V), (uint16_t*)d_hidden + t0 * H,
-                          st);
+    rc = launch_bwd_chunk(c.stash, lm_head_t, ids, shift, t0, n, S, V, H, lse + t0,
+                          grad_logprob + t0, c.bwd, (uint16_t*)d_hidden + t0 * H, st);
     if (rc) return rc;
   }
   return ARTK_OK;
@@ -799,13 +885,9 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
 
 size_t artk_grpo_fused_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {
   Workspace ws(nullptr, 0);
-  uint16_t* stash;
-  float2* part;
-  float *sel, *partial, *lse, *coef, *pl, *kl;
-  int nsplit, *count;
-  int64_t Tc = clamp_chunk(T, chunk_tokens);
-  return chunk_workspace(T, V, H, Tc, true, ws, &stash, &part, &sel, &partial, &nsplit, &lse, &coef,
-                         &pl, &kl, &count);
+  ChunkScratch c;
+  carve(ws, T, V, H, clamp_chunk(T, V, chunk_tokens), true, c);
+  return ws.used + 256;
 }
 
 int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_head_t,
@@ -822,26 +904,22 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
                  "null pointer argument");
   ARTK_CHECK_ARG(aligned16(lm_head_t) && aligned16(d_hidden), "pointers must be 16-byte aligned");
   ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
-  const int64_t Tc = clamp_chunk(T, chunk_tokens);
+  const int64_t Tc = clamp_chunk(T, V, chunk_tokens);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* stash;
-  float2* part;
-  float *sel, *partial, *lse, *coef, *pl, *kl;
-  int nsplit, *count;
-  chunk_workspace(T, V, H, Tc, true, ws, &stash, &part, &sel, &partial, &nsplit, &lse, &coef, &pl,
-                  &kl, &count);
+  ChunkScratch c;
+  carve(ws, T, V, H, Tc, true, c);
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
   const float* ref = (beta > 0.f) ? ref_logprob : nullptr;
-  mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, 1, count);
+  mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, 1, c.count);
   ARTK_CHECK_LAUNCH();
   for (int64_t t0 = 0; t0 < T; t0 += Tc) {
     const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
-    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, t0, n, T, S, V, H, part, sel, stash,
-                          logprob + t0, lse + t0, st);
+    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, t0, n, T, S, V, H, c.part, c.sel, c.stash,
+                          logprob + t0, c.lse + t0, st);
     if (rc) return rc;
     LossParams p;
     p.new_lp = logprob + t0;
@@ -850,7 +928,7 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
     p.mask = mask;
     p.weights = weights;
     p.ref_lp = ref ? ref + t0 : nullptr;
-    p.count = count;
+    p.count = c.count;
     p.t0 = t0;
     p.n = n;
     p.T = T;
@@ -859,16 +937,16 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
     p.clip_lo = clip_lo;
     p.clip_hi = clip_hi;
     p.beta = beta;
-    p.pl_tok = pl + t0;
-    p.kl_tok = kl + t0;
-    p.coef = coef + t0;
+    p.pl_tok = c.pl + t0;
+    p.kl_tok = c.kl + t0;
+    p.coef = c.coef + t0;
     grpo_loss_tok_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(p);
     ARTK_CHECK_LAUNCH();
-    rc = launch_bwd_chunk(stash, lm_head_t, tokens, 1, t0, n, S, V, H, lse + t0, coef + t0, partial,
-                          chunk_nsplit(n, Tc, nsplit, H, V), (uint16_t*)d_hidden + t0 * H, st);
+    rc = launch_bwd_chunk(c.stash, lm_head_t, tokens, 1, t0, n, S, V, H, c.lse + t0, c.coef + t0,
+                          c.bwd, (uint16_t*)d_hidden + t0 * H, st);
     if (rc) return rc;
   }
-  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, ref ? beta : 0.f, scalars);
+  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(c.pl, c.kl, T, c.count, ref ? beta : 0.f, scalars);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

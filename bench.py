@@ -124,14 +124,17 @@ def main():
 
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T / (dt / args.steps)
-    alg_flops_step = 4.0 * T * V * H
+    # rows whose loss coefficient is zero (non-assistant positions) have a zero d_hidden row
+    # and are skipped by the backward: the algorithmic work counts them in the forward only
+    t_active = int(out[0][3].item())
+    alg_flops_step = 2.0 * T * V * H + 2.0 * t_active * V * H
     # dominant kernel: one launch covers `chunk` positions against the whole vocabulary
     fwd_launch_ms = fwd_ms / max(fwd_n, 1)
     launches_per_step = fwd_n / args.steps
     flops_per_launch = 2.0 * T * V * H / launches_per_step
     achieved = flops_per_launch / (fwd_launch_ms * 1e-3) / 1e12
     bwd_launch_ms = bwd_ms / max(bwd_n, 1)
-    bwd_achieved = (2.0 * T * V * H / (bwd_n / args.steps)) / (bwd_launch_ms * 1e-3) / 1e12
+    bwd_achieved = (2.0 * t_active * V * H / (bwd_n / args.steps)) / (bwd_launch_ms * 1e-3) / 1e12
 
     result = {
         "metric": "GRPO loss fwd+bwd tokens/sec @Qwen2.5-7B shape" if args.workload == "c3"
@@ -148,7 +151,9 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": case.name, "tokens": T, "hidden": H, "vocab": V,
-                   "chunk_tokens": chunk, "mask_fraction": float(case.assistant_mask.float().mean())},
+                   "chunk_tokens": chunk, "mask_fraction": float(case.assistant_mask.float().mean()),
+                   "t_active": t_active},
+        "algorithmic_flops_per_step": alg_flops_step,
         "tflops_algorithmic": alg_flops_step / (dt / args.steps) / 1e12,
         "frac_of_bf16_peak": alg_flops_step / (dt / args.steps) / 1e12 / PEAK_BF16_TFLOPS,
         "roofline": {

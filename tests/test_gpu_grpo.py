@@ -157,6 +157,31 @@ def test_fused_is_deterministic(artk_lib, gpu):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("density", [0.0, 1.0])
+def test_fused_all_or_no_rows_active(artk_lib, gpu, density):
+    """Edge cases of the active-row compaction: empty mask (zero loss, zero
+    gradient, no GEMM work) and a mask covering every position."""
+    T, H, V = 512, 128, 4096
+    case = synthetic.make_grpo_case("t", 17, T, H, V, 4, 4, 0.5)
+    case.assistant_mask = torch.full_like(case.assistant_mask, bool(density))
+    from art_amd.advantage import token_weights
+    case.weights = token_weights(case.assistant_mask, case.traj_id) if density else torch.zeros_like(case.weights)
+    ref = oracle_case(case, 256)
+    hidden = case.hidden.to(gpu).requires_grad_(True)
+    loss, metrics, logprob = fused_grpo_loss(
+        hidden, case.lm_head.to(gpu), case.tokens.to(gpu), case.logprobs.to(gpu),
+        case.advantages.to(gpu), case.assistant_mask.to(gpu), case.weights.to(gpu), chunk_tokens=256)
+    loss.backward()
+    assert (logprob.cpu() - ref["logprobs"]).abs().max().item() <= LP_TOL
+    if density == 0.0:
+        assert loss.item() == 0.0 and hidden.grad.abs().max().item() == 0.0
+        assert metrics["mask_count"].item() == 0
+    else:
+        assert abs(loss.item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item())
+        assert rel_l2(hidden.grad.float().cpu(), ref["d_hidden"]) <= GRAD_TOL
+        assert metrics["mask_count"].item() == T - 1  # the last position's mask shifts out
+
+
 def test_config1_full_size(artk_lib, gpu):
     """BASELINE config 1 (Qwen2.5-0.5B shape) at full size against the oracle."""
     print("config1 full size", flush=True)
