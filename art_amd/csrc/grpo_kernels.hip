@@ -48,6 +48,7 @@ struct FwdParams {
   float2* part;         // [2*VT][Tc]  (max, sumexp)
   float* sel;           // [Tc]        selected logit (pre-filled with NaN)
   uint16_t* stash;      // [Tc,V] bf16 logits or nullptr
+  const uint8_t* need;  // [Tc] rows of the stash that the backward will read
   int VT, TT;
 };
 
@@ -81,7 +82,9 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
   if (STASH) {
 #pragma unroll
     for (int ni = 0; ni < 4; ++ni) {
-      if (col[ni] < p.Tc) {
+      const bool want = col[ni] < p.Tc && p.need[col[ni]] != 0;
+      if (!__any(want)) continue;
+      if (want) {
         uint16_t* row = p.stash + (int64_t)col[ni] * p.V;
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi)
@@ -187,6 +190,29 @@ __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restr
     lse[t] = z;
     logprob[t] = sel[t] - z;
   }
+}
+
+// need[i] = 1 when position t0+i can have a non-zero loss coefficient: its
+// (shifted) mask is set and weight and advantage are non-zero.
+__global__ __launch_bounds__(256) void need_from_inputs_kernel(const uint8_t* __restrict__ mask,
+                                                               const float* __restrict__ weights,
+                                                               const float* __restrict__ adv,
+                                                               const float* __restrict__ ref_lp,
+                                                               int64_t t0, int64_t n, int64_t S,
+                                                               int shift, uint8_t* __restrict__ need) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  int64_t src;
+  uint8_t v = 0;
+  if (shifted_index(t0 + i, S, shift, src))
+    v = mask[src] != 0 && weights[src] != 0.f && (adv[src] != 0.f || ref_lp != nullptr);
+  need[i] = v;
+}
+
+__global__ __launch_bounds__(256) void need_from_grad_kernel(const float* __restrict__ g, int64_t n,
+                                                             uint8_t* __restrict__ need) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) need[i] = g[i] != 0.f;
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -624,7 +650,8 @@ static int32_t check_common(const void* hidden, const void* lm_head, int64_t T, 
 static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const int64_t* ids,
                                 int shift, int64_t t0, int64_t Tc, int64_t T, int64_t S, int64_t V,
                                 int64_t H, float2* part, float* sel, uint16_t* stash,
-                                float* logprob_chunk, float* lse_chunk, hipStream_t st) {
+                                const uint8_t* need, float* logprob_chunk, float* lse_chunk,
+                                hipStream_t st) {
   FwdParams p;
   p.hidden = (const char*)hidden + t0 * H * 2;
   p.W = lm_head;
@@ -639,6 +666,7 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   p.part = part;
   p.sel = sel;
   p.stash = stash;
+  p.need = need;
   p.VT = (int)((V + TILE - 1) / TILE);
   p.TT = (int)((Tc + TILE - 1) / TILE);
   fill_f32_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(sel, Tc, NAN);
@@ -741,8 +769,8 @@ int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t*
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
-  return launch_fwd_chunk(hidden, lm_head, ids, shift, 0, T, T, S, V, H, part, sel, nullptr, logprob,
-                          lse, (hipStream_t)stream);
+  return launch_fwd_chunk(hidden, lm_head, ids, shift, 0, T, T, S, V, H, part, sel, nullptr, nullptr,
+                          logprob, lse, (hipStream_t)stream);
 }
 
 // Scratch of one chunk of Tc positions carved out of the caller's workspace.
@@ -750,6 +778,7 @@ struct ChunkScratch {
   uint16_t* stash;  // [Tc,V] bf16 logits, then softmax gradient
   float2* part;     // [2*VT][Tc]
   float* sel;       // [Tc]
+  uint8_t* need;    // [Tc]
   BwdScratch bwd;
   float *lse, *coef, *pl, *kl;  // [T] each (fused op only)
   int* count;
@@ -762,6 +791,7 @@ static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bo
   c.stash = ws.take<uint16_t>((size_t)(Tc * V));
   c.part = ws.take<float2>((size_t)(2 * VT * Tc));
   c.sel = ws.take<float>((size_t)Tc);
+  c.need = ws.take<uint8_t>((size_t)Tc);
   c.bwd.part_rows = bwd_part_rows(Tc, H, V);
   c.bwd.partial = ws.take<float>((size_t)c.bwd.part_rows * H);
   c.bwd.active_idx = ws.take<int>((size_t)Tc);
@@ -818,8 +848,10 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
   for (int64_t t0 = 0; t0 < T; t0 += Tc) {
     const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
     // The scratch row pitch is V, so a shorter last chunk simply uses fewer rows.
+    need_from_grad_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(grad_logprob + t0, n, c.need);
+    ARTK_CHECK_LAUNCH();
     rc = launch_fwd_chunk(hidden, lm_head, ids, shift, t0, n, T, S, V, H, c.part, c.sel, c.stash,
-                          c.lp_tmp, c.lse_tmp, st);
+                          c.need, c.lp_tmp, c.lse_tmp, st);
     if (rc) return rc;
     rc = launch_bwd_chunk(c.stash, lm_head_t, ids, shift, t0, n, S, V, H, lse + t0,
                           grad_logprob + t0, c.bwd, (uint16_t*)d_hidden + t0 * H, st);
@@ -918,8 +950,11 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
   ARTK_CHECK_LAUNCH();
   for (int64_t t0 = 0; t0 < T; t0 += Tc) {
     const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
+    need_from_inputs_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(mask, weights, advantages,
+                                                                         ref, t0, n, S, 1, c.need);
+    ARTK_CHECK_LAUNCH();
     rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, t0, n, T, S, V, H, c.part, c.sel, c.stash,
-                          logprob + t0, c.lse + t0, st);
+                          c.need, logprob + t0, c.lse + t0, st);
     if (rc) return rc;
     LossParams p;
     p.new_lp = logprob + t0;
