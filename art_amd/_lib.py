@@ -47,6 +47,16 @@ SIGNATURES = {
     "artk_lora_linear_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "artk_lora_linear_bwd": (
         _i32, [_p, _p, _p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),
+    "artk_moe_route_workspace_bytes": (_sz, [_i64, _i32, _i32]),
+    "artk_moe_route": (_i32, [_p, _i64, _i32, _i32, _p, _p, _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "artk_moe_lora_grouped_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, _i32]),
+    "artk_moe_lora_grouped_fwd": (
+        _i32, [_p, _p, _p, _p, _p, _f32, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _p, _p, _sz, _p]),
+    "artk_moe_lora_grouped_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, _i32]),
+    "artk_moe_lora_grouped_bwd": (
+        _i32, [_p, _p, _p, _p, _p, _p, _p, _f32, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _p, _p,
+               _p, _sz, _p]),
+    "artk_transpose_bf16_batched": (_i32, [_p, _p, _i64, _i64, _i64, _p]),
     "artk_profile_enable": (_i32, [_i32]),
     "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
 }

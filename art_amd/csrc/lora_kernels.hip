@@ -15,6 +15,7 @@
 // dA, dB: reductions along the token axis) are bandwidth-bound helpers.
 #include "common.hpp"
 #include "gemm_nt.hpp"
+#include "lora_common.hpp"
 
 namespace artk {
 
@@ -206,25 +207,6 @@ __global__ __launch_bounds__(256) void coldot_reduce_kernel(const float* __restr
   }
 }
 
-// dst [R1,C1] bf16 = zero-padded copy of src [R0,C0] (or of its transpose).
-__global__ __launch_bounds__(256) void pad_copy_bf16_kernel(const uint16_t* __restrict__ src,
-                                                            int64_t R0, int64_t C0, int transpose,
-                                                            uint16_t* __restrict__ dst, int64_t R1,
-                                                            int64_t C1) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= R1 * C1) return;
-  const int64_t r = i / C1, c = i - r * C1;
-  uint16_t v = 0;
-  if (!transpose) {
-    if (r < R0 && c < C0) v = src[r * C0 + c];
-  } else {
-    if (c < R0 && r < C0) v = src[c * C0 + r];
-  }
-  dst[i] = v;
-}
-
-static int round16(int r) { return (r + 15) / 16 * 16; }
-
 static int32_t check_lora(int64_t T, int64_t in, int64_t out, int r) {
   ARTK_CHECK_ARG(T > 0 && in > 0 && out > 0 && r > 0, "T, in, out, r must be positive");
   if (in % BK != 0 || out % BK != 0) {
@@ -235,15 +217,6 @@ static int32_t check_lora(int64_t T, int64_t in, int64_t out, int r) {
     set_error("LoRA rank %d must be a multiple of 8 and at most 64", r);
     return ARTK_ERR_UNSUPPORTED_SHAPE;
   }
-  return ARTK_OK;
-}
-
-static int32_t launch_pad(const void* src, int64_t R0, int64_t C0, int transpose, uint16_t* dst,
-                          int64_t R1, int64_t C1, hipStream_t st) {
-  const int64_t n = R1 * C1;
-  pad_copy_bf16_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint16_t*)src, R0, C0,
-                                                                    transpose, dst, R1, C1);
-  ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
 
@@ -327,8 +300,8 @@ int32_t artk_lora_linear_fwd(const void* x, const void* W, const void* A, const 
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(A, r, in, 0, A16, RP, in, st))) return rc;
-  if ((rc = launch_pad(B, out, r, 0, B16, out, RP, st))) return rc;
+  if ((rc = launch_pad(A, 1, r, in, 0, A16, RP, in, st))) return rc;
+  if ((rc = launch_pad(B, 1, out, r, 0, B16, out, RP, st))) return rc;
   if ((rc = launch_rowdot(x, A16, T, in, r, RP, scale, xa, xa16, st))) return rc;
   return launch_lora_gemm(W, x, B16, xa16, y, out, T, in, RP, st);
 }
@@ -367,8 +340,8 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(B, out, r, 1, Bt16, RP, out, st))) return rc;
-  if ((rc = launch_pad(A, r, in, 1, At16, in, RP, st))) return rc;
+  if ((rc = launch_pad(B, 1, out, r, 1, Bt16, RP, out, st))) return rc;
+  if ((rc = launch_pad(A, 1, r, in, 1, At16, in, RP, st))) return rc;
   // g B  -> gb (f32) and s * gb (bf16, padded)
   if ((rc = launch_rowdot(g, Bt16, T, out, r, RP, scale, gb, gb16, st))) return rc;
   // dx = g W + (s g B) A

@@ -1,0 +1,577 @@
+// MoE expert path for gfx950: router top-k, stable expert-contiguous
+// permutation, and per-expert LoRA linears as grouped GEMMs
+//   y[i,:] = x[row(i),:] W_e^T + s (x[row(i),:] A_e^T) B_e^T      e = expert of row i
+// over the permuted (token, expert) rows, with their backward.
+//
+// The reference has no MoE code at this commit; the contract comes from the
+// benchmark configuration (128 experts, top-8, Qwen3-30B-A3B-style expert
+// shapes, rank-8 LoRA per expert).  Routing follows the usual definition
+// (softmax over router logits in fp32, top-k, renormalise); the selection is
+// made on the logits, which order like the softmax, ties to the lower expert
+// index, and the permutation is the stable sort of the token-major (token, slot)
+// list by expert id, so both integer outputs are reproducible bit for bit.
+#include "common.hpp"
+#include "gemm_nt.hpp"
+#include "lora_common.hpp"
+
+#include <math.h>
+
+namespace artk {
+
+// ----------------------------------------------------------------------------
+// Routing: one wavefront per token.
+// ----------------------------------------------------------------------------
+constexpr int MOE_MAX_E = 256;
+constexpr int MOE_MAX_K = 16;
+
+__global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ logits, int64_t T,
+                                                       int E, int k, int* __restrict__ topk_idx,
+                                                       float* __restrict__ topk_w) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  float x[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = lane + 64 * i;
+    x[i] = e < E ? logits[t * E + e] : -INFINITY;
+  }
+  float m = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+  m = wave_max(m);
+  float myp = 0.f;  // lane j keeps the probability mass of slot j
+  float psum = 0.f;
+  for (int j = 0; j < k; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (x[i] > bv) {
+        bv = x[i];
+        bi = lane + 64 * i;
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (lane + 64 * i == bi) x[i] = -INFINITY;
+    const float pj = expf(bv - m);
+    psum += pj;
+    if (lane == j) myp = pj;
+    if (lane == 0) topk_idx[t * k + j] = bi;
+  }
+  if (lane < k) topk_w[t * k + lane] = myp / psum;
+}
+
+// ----------------------------------------------------------------------------
+// Stable counting sort of the n = T*k keys (expert ids) in chunks of 1024.
+// ----------------------------------------------------------------------------
+constexpr int PERM_CHUNK = 1024;
+
+__global__ __launch_bounds__(PERM_CHUNK) void moe_hist_kernel(const int* __restrict__ keys, int n,
+                                                              int E, int* __restrict__ cnt) {
+  __shared__ int hist[MOE_MAX_E];
+  for (int i = threadIdx.x; i < E; i += PERM_CHUNK) hist[i] = 0;
+  __syncthreads();
+  const int f = blockIdx.x * PERM_CHUNK + threadIdx.x;
+  if (f < n) atomicAdd(&hist[keys[f]], 1);
+  __syncthreads();
+  for (int i = threadIdx.x; i < E; i += PERM_CHUNK) cnt[blockIdx.x * E + i] = hist[i];
+}
+
+// offsets[e]: first sorted position of expert e; base[b][e]: first sorted
+// position of chunk b's entries of expert e; tile_prefix / blk_prefix: prefix
+// sums of ceil(rows_e / 256) and ceil(rows_e / 16) (work lists of the grouped
+// kernels).  One block of 256 threads.
+__global__ __launch_bounds__(256) void moe_scan_kernel(const int* __restrict__ cnt, int nb, int E,
+                                                       int* __restrict__ offsets,
+                                                       int* __restrict__ base,
+                                                       int* __restrict__ tile_prefix,
+                                                       int* __restrict__ blk_prefix) {
+  __shared__ int tot[MOE_MAX_E];
+  __shared__ int off[MOE_MAX_E + 1];
+  const int e = threadIdx.x;
+  if (e < E) {
+    int s = 0;
+    for (int b = 0; b < nb; ++b) s += cnt[b * E + e];
+    tot[e] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, tp = 0, bp = 0;
+    for (int i = 0; i < E; ++i) {
+      off[i] = run;
+      offsets[i] = run;
+      tile_prefix[i] = tp;
+      blk_prefix[i] = bp;
+      run += tot[i];
+      tp += (tot[i] + TILE - 1) / TILE;
+      bp += (tot[i] + 15) / 16;
+    }
+    off[E] = run;
+    offsets[E] = run;
+    tile_prefix[E] = tp;
+    blk_prefix[E] = bp;
+  }
+  __syncthreads();
+  if (e < E) {
+    int run = off[e];
+    for (int b = 0; b < nb; ++b) {
+      base[b * E + e] = run;
+      run += cnt[b * E + e];
+    }
+  }
+}
+
+__global__ __launch_bounds__(PERM_CHUNK) void moe_scatter_kernel(const int* __restrict__ keys, int n,
+                                                                 int E, int k,
+                                                                 const int* __restrict__ base,
+                                                                 int* __restrict__ perm,
+                                                                 int* __restrict__ inv_perm,
+                                                                 int* __restrict__ row_token) {
+  __shared__ int ks[PERM_CHUNK];
+  const int f = blockIdx.x * PERM_CHUNK + threadIdx.x;
+  const int key = f < n ? keys[f] : -1;
+  ks[threadIdx.x] = key;
+  __syncthreads();
+  int rank = 0;
+  for (int j = 0; j < PERM_CHUNK; ++j) rank += (j < (int)threadIdx.x && ks[j] == key) ? 1 : 0;
+  if (f < n) {
+    const int pos = base[blockIdx.x * E + key] + rank;
+    perm[pos] = f;
+    inv_perm[f] = pos;
+    row_token[pos] = f / k;
+  }
+}
+
+// Largest g with prefix[g] <= x, for a non-decreasing prefix[0..G] with prefix[G] > x.
+__device__ __forceinline__ int find_group(const int* __restrict__ prefix, int G, int x) {
+  int lo = 0, hi = G;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (prefix[mid] <= x) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ----------------------------------------------------------------------------
+// Grouped GEMM: 256-row tiles never straddle experts.
+// ----------------------------------------------------------------------------
+struct MoeGemmParams {
+  const void* W;           // [E,M,K] bf16
+  const void* X;           // activations, [*,K] bf16
+  const int* gather;       // permuted row i reads X row gather[i]; nullptr: row i
+  const uint16_t* Pe;      // [E,M,RP] padded low-rank factor of the weights
+  const uint16_t* Qe;      // [n_rows,RP] padded, scaled low-rank activations
+  uint16_t* out;           // [n_rows,M]
+  const int* offsets;      // [E+1]
+  const int* tile_prefix;  // [E+1]
+  int64_t M, K;
+  int E, RP, MT;
+};
+
+__global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int n_work = p.tile_prefix[p.E] * p.MT;
+  if ((int)blockIdx.x >= n_work) return;
+  const int id = xcd_remap(blockIdx.x, n_work);
+  const int rt = id / p.MT, mt = id - rt * p.MT;
+  const int e = find_group(p.tile_prefix, p.E, rt);
+  const int64_t row0 = p.offsets[e] + (int64_t)(rt - p.tile_prefix[e]) * TILE;
+  const int64_t row_end = p.offsets[e + 1];
+  const int nvalid = (int)(row_end - row0 < TILE ? row_end - row0 : TILE);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5;
+
+  TileAcc acc;
+  acc.zero();
+  gemm_tile_nt(acc, smem, (const char*)p.W + (int64_t)e * p.M * p.K * 2, p.K, (int64_t)mt * TILE, p.M,
+               p.X, p.K, row0, row_end, 0, (int)p.K, p.gather);
+
+  if (p.Pe != nullptr) {
+    const uint16_t* pe = p.Pe + (int64_t)e * p.M * p.RP;
+    int64_t prow[4], qrow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
+      prow[i] = r < p.M ? r : p.M - 1;
+      int c = wn * 128 + i * 32 + (lane & 31);
+      qrow[i] = row0 + (c < nvalid ? c : nvalid - 1);
+    }
+    for (int e0 = 0; e0 < p.RP; e0 += 16) {
+      Frags f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        f.p[i] = *(const bf16x8*)(pe + prow[i] * p.RP + e0 + half * 8);
+        f.q[i] = *(const bf16x8*)(p.Qe + qrow[i] * p.RP + e0 + half * 8);
+      }
+      mma_frags(acc, f);
+    }
+  }
+
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    const int c = acc_col(wn, ni, lane);
+    if (c >= nvalid) continue;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
+        if (m >= p.M) continue;
+        bf16x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = (__bf16)acc.c[mi][ni][q * 4 + k];
+        *(bf16x4*)(p.out + (row0 + c) * p.M + m) = o;
+      }
+  }
+}
+
+// Grouped row products: 16-row blocks never straddle experts.
+//   out[i, j] = sum_k X[row(i), k] Mt_e[j, k]
+__global__ __launch_bounds__(256) void moe_rowdot16_kernel(
+    const uint16_t* __restrict__ X, const int* __restrict__ gather, const uint16_t* __restrict__ Mt,
+    const int* __restrict__ offsets, const int* __restrict__ blk_prefix, int E, int64_t K, int R,
+    int RP, float scale, float* __restrict__ out_f32, uint16_t* __restrict__ out_bf16) {
+  __shared__ floatx4 red[3][64];
+  const int b = blockIdx.x;
+  if (b >= blk_prefix[E]) return;
+  const int e = find_group(blk_prefix, E, b);
+  const int64_t row0 = offsets[e] + (int64_t)(b - blk_prefix[e]) * 16;
+  const int64_t row_end = offsets[e + 1];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j0 = blockIdx.y * 16;
+  int64_t row = row0 + (lane & 15);
+  if (row >= row_end) row = row_end - 1;
+  const int64_t src = gather ? gather[row] : row;
+  const uint16_t* xp = X + src * K + (lane >> 4) * 8;
+  const uint16_t* mp = Mt + ((int64_t)e * RP + j0 + (lane & 15)) * K + (lane >> 4) * 8;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int64_t k = (int64_t)wave * 32; k < K; k += 128) {
+    bf16x8 a = *(const bf16x8*)(xp + k);
+    bf16x8 bb = *(const bf16x8*)(mp + k);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bb, acc, 0, 0, 0);
+  }
+  if (wave > 0) red[wave - 1][lane] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    acc += red[0][lane];
+    acc += red[1][lane];
+    acc += red[2][lane];
+    const int j = j0 + (lane & 15);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t i = row0 + (lane >> 4) * 4 + q;
+      if (i < row_end) {
+        if (j < R) out_f32[i * R + j] = acc[q];
+        out_bf16[i * RP + j] = f32_to_bf16(acc[q] * scale);
+      }
+    }
+  }
+}
+
+// Grouped column products over the rows of one expert:
+//   out_e[c, r] = scale * sum_{i in rows(e)} X[row(i), c] Y[i, r]    r in [r0, r0+8)
+// out is [E,C,R], or [E,R,C] when transpose_out.  Fixed summation order.
+__global__ __launch_bounds__(256) void moe_coldot8_kernel(
+    const uint16_t* __restrict__ X, const int* __restrict__ gather, const float* __restrict__ Y,
+    const int* __restrict__ offsets, int64_t C, int R, float scale, int transpose_out,
+    float* __restrict__ out) {
+  __shared__ float ys[128][8];
+  __shared__ int rows[128];
+  const int64_t c = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int e = blockIdx.y;
+  const int r0 = blockIdx.z * 8;
+  const int64_t begin = offsets[e], end = offsets[e + 1];
+  float acc[4][8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc[j][q] = 0.f;
+  for (int64_t s0 = begin; s0 < end; s0 += 128) {
+    const int nrows = (int)(end - s0 < 128 ? end - s0 : 128);
+    __syncthreads();
+    for (int i = threadIdx.x; i < 128 * 8; i += 256) {
+      const int rr = i >> 3, q = i & 7;
+      ys[rr][q] = rr < nrows ? Y[(s0 + rr) * R + r0 + q] : 0.f;
+    }
+    if (threadIdx.x < 128) {
+      const int64_t i = s0 + threadIdx.x;
+      rows[threadIdx.x] = threadIdx.x < nrows ? (gather ? gather[i] : (int)i) : 0;
+    }
+    __syncthreads();
+    if (c < C) {
+      for (int rr = 0; rr < nrows; ++rr) {
+        const uint2 raw = *(const uint2*)(X + (int64_t)rows[rr] * C + c);
+        const float x0 = __uint_as_float(raw.x << 16), x1 = __uint_as_float(raw.x & 0xffff0000u);
+        const float x2 = __uint_as_float(raw.y << 16), x3 = __uint_as_float(raw.y & 0xffff0000u);
+        const floatx4 ya = *(const floatx4*)&ys[rr][0];
+        const floatx4 yb = *(const floatx4*)&ys[rr][4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc[0][q] += x0 * ya[q];
+          acc[1][q] += x1 * ya[q];
+          acc[2][q] += x2 * ya[q];
+          acc[3][q] += x3 * ya[q];
+          acc[0][4 + q] += x0 * yb[q];
+          acc[1][4 + q] += x1 * yb[q];
+          acc[2][4 + q] += x2 * yb[q];
+          acc[3][4 + q] += x3 * yb[q];
+        }
+      }
+    }
+  }
+  if (c >= C) return;
+  float* oe = out + (int64_t)e * C * R;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float v = acc[j][q] * scale;
+      if (transpose_out)
+        oe[(int64_t)(r0 + q) * C + c + j] = v;
+      else
+        oe[(c + j) * R + r0 + q] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void transpose_bf16_batched_kernel(const uint16_t* __restrict__ in,
+                                                                     uint16_t* __restrict__ out,
+                                                                     int64_t R, int64_t C) {
+  __shared__ uint16_t tile[64][66];
+  in += (int64_t)blockIdx.z * R * C;
+  out += (int64_t)blockIdx.z * R * C;
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    int64_t r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? in[r * C + c] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int64_t c = c0 + i, r = r0 + tx;
+    if (c < C && r < R) out[c * R + r] = tile[tx][i];
+  }
+}
+
+static int32_t check_moe(int64_t n_rows, int64_t in, int64_t out, int E, int r) {
+  ARTK_CHECK_ARG(n_rows > 0 && in > 0 && out > 0 && E > 0 && r > 0, "sizes must be positive");
+  if (in % BK != 0 || out % BK != 0) {
+    set_error("in (%lld) and out (%lld) must be multiples of %d", (long long)in, (long long)out, BK);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  if (r % 8 != 0 || r > 64 || E > MOE_MAX_E) {
+    set_error("LoRA rank must be a multiple of 8 and <= 64, experts <= %d", MOE_MAX_E);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  if (n_rows >= (1ll << 31) / 8) {
+    set_error("too many rows");
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  return ARTK_OK;
+}
+
+static int32_t launch_moe_gemm(const void* W, const void* X, const int* gather, const uint16_t* Pe,
+                               const uint16_t* Qe, void* out, const int* offsets,
+                               const int* tile_prefix, int64_t n_rows, int64_t M, int64_t K, int E,
+                               int RP, hipStream_t st) {
+  MoeGemmParams p;
+  p.W = W;
+  p.X = X;
+  p.gather = gather;
+  p.Pe = Pe;
+  p.Qe = Qe;
+  p.out = (uint16_t*)out;
+  p.offsets = offsets;
+  p.tile_prefix = tile_prefix;
+  p.M = M;
+  p.K = K;
+  p.E = E;
+  p.RP = RP;
+  p.MT = (int)((M + TILE - 1) / TILE);
+  const int64_t max_row_tiles = (n_rows + TILE - 1) / TILE + E;
+  prof_begin(PROF_MOE_GEMM, st);
+  moe_gemm_kernel<<<(unsigned)(max_row_tiles * p.MT), NTHREADS, 0, st>>>(p);
+  prof_end(PROF_MOE_GEMM, st);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+static int32_t launch_moe_rowdot(const void* X, const int* gather, const uint16_t* Mt,
+                                 const int* offsets, const int* blk_prefix, int64_t n_rows, int E,
+                                 int64_t K, int R, int RP, float scale, float* out_f32,
+                                 uint16_t* out_bf16, hipStream_t st) {
+  dim3 grid((unsigned)((n_rows + 15) / 16 + E), (unsigned)(RP / 16));
+  moe_rowdot16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, gather, Mt, offsets, blk_prefix, E, K,
+                                            R, RP, scale, out_f32, out_bf16);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+static int32_t launch_moe_coldot(const void* X, const int* gather, const float* Y, const int* offsets,
+                                 int E, int64_t C, int R, float scale, int transpose_out, float* out,
+                                 hipStream_t st) {
+  dim3 grid((unsigned)((C / 4 + 255) / 256), (unsigned)E, (unsigned)(R / 8));
+  moe_coldot8_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, gather, Y, offsets, C, R, scale,
+                                           transpose_out, out);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+}  // namespace artk
+
+using namespace artk;
+
+extern "C" {
+
+size_t artk_moe_route_workspace_bytes(int64_t T, int32_t E, int32_t k) {
+  Workspace ws(nullptr, 0);
+  const int64_t n = T * k;
+  const int64_t nb = (n + PERM_CHUNK - 1) / PERM_CHUNK;
+  ws.take<int>((size_t)(nb * E));
+  ws.take<int>((size_t)(nb * E));
+  return ws.used + 256;
+}
+
+int32_t artk_moe_route(const float* router_logits, int64_t T, int32_t E, int32_t k, int32_t* topk_idx,
+                       float* topk_w, int32_t* perm, int32_t* inv_perm, int32_t* row_token,
+                       int32_t* expert_offsets, int32_t* tile_prefix, int32_t* blk_prefix,
+                       void* workspace, size_t workspace_bytes, artk_stream_t stream) {
+  ARTK_CHECK_ARG(router_logits && topk_idx && topk_w && perm && inv_perm && row_token &&
+                     expert_offsets && tile_prefix && blk_prefix,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(T > 0 && E > 0 && k > 0 && k <= E, "T, E, k must be positive and k <= E");
+  if (E > MOE_MAX_E || k > MOE_MAX_K || T * k >= (1ll << 30)) {
+    set_error("supported: experts <= %d, top-k <= %d", MOE_MAX_E, MOE_MAX_K);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  const int n = (int)(T * k);
+  const int nb = (n + PERM_CHUNK - 1) / PERM_CHUNK;
+  Workspace ws(workspace, workspace_bytes);
+  int* cnt = ws.take<int>((size_t)nb * E);
+  int* base = ws.take<int>((size_t)nb * E);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  moe_topk_kernel<<<(unsigned)((T + 3) / 4), 256, 0, st>>>(router_logits, T, E, k, topk_idx, topk_w);
+  ARTK_CHECK_LAUNCH();
+  moe_hist_kernel<<<nb, PERM_CHUNK, 0, st>>>(topk_idx, n, E, cnt);
+  ARTK_CHECK_LAUNCH();
+  moe_scan_kernel<<<1, 256, 0, st>>>(cnt, nb, E, expert_offsets, base, tile_prefix, blk_prefix);
+  ARTK_CHECK_LAUNCH();
+  moe_scatter_kernel<<<nb, PERM_CHUNK, 0, st>>>(topk_idx, n, E, k, base, perm, inv_perm, row_token);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+size_t artk_moe_lora_grouped_fwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
+                                                 int32_t r) {
+  const int RP = round16(r);
+  Workspace ws(nullptr, 0);
+  ws.take<uint16_t>((size_t)E * RP * in);
+  ws.take<uint16_t>((size_t)E * out * RP);
+  ws.take<uint16_t>((size_t)n_rows * RP);
+  return ws.used + 256;
+}
+
+int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const void* W, const void* A,
+                                  const void* B, float scale, const int32_t* expert_offsets,
+                                  const int32_t* tile_prefix, const int32_t* blk_prefix,
+                                  int64_t n_rows, int64_t in, int64_t out, int32_t E, int32_t r,
+                                  void* y, float* xa, void* workspace, size_t workspace_bytes,
+                                  artk_stream_t stream) {
+  int32_t rc = check_moe(n_rows, in, out, E, r);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(x && W && A && B && expert_offsets && tile_prefix && blk_prefix && y && xa,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(y), "pointers must be 16-byte aligned");
+  const int RP = round16(r);
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* A16 = ws.take<uint16_t>((size_t)E * RP * in);
+  uint16_t* B16 = ws.take<uint16_t>((size_t)E * out * RP);
+  uint16_t* xa16 = ws.take<uint16_t>((size_t)n_rows * RP);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = launch_pad(A, E, r, in, 0, A16, RP, in, st))) return rc;
+  if ((rc = launch_pad(B, E, out, r, 0, B16, out, RP, st))) return rc;
+  if ((rc = launch_moe_rowdot(x, gather, A16, expert_offsets, blk_prefix, n_rows, E, in, r, RP, scale,
+                              xa, xa16, st)))
+    return rc;
+  return launch_moe_gemm(W, x, gather, B16, xa16, y, expert_offsets, tile_prefix, n_rows, out, in, E,
+                         RP, st);
+}
+
+size_t artk_moe_lora_grouped_bwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
+                                                 int32_t r) {
+  const int RP = round16(r);
+  Workspace ws(nullptr, 0);
+  ws.take<uint16_t>((size_t)E * RP * out);
+  ws.take<uint16_t>((size_t)E * in * RP);
+  ws.take<float>((size_t)n_rows * r);
+  ws.take<uint16_t>((size_t)n_rows * RP);
+  return ws.used + 256;
+}
+
+int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* gather, const void* W_t,
+                                  const void* A, const void* B, const float* xa, float scale,
+                                  const int32_t* expert_offsets, const int32_t* tile_prefix,
+                                  const int32_t* blk_prefix, int64_t n_rows, int64_t in, int64_t out,
+                                  int32_t E, int32_t r, void* dx, float* dA, float* dB,
+                                  void* workspace, size_t workspace_bytes, artk_stream_t stream) {
+  int32_t rc = check_moe(n_rows, in, out, E, r);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(g && x && W_t && A && B && xa && expert_offsets && tile_prefix && blk_prefix && dx &&
+                     dA && dB,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(dx),
+                 "pointers must be 16-byte aligned");
+  const int RP = round16(r);
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* Bt16 = ws.take<uint16_t>((size_t)E * RP * out);
+  uint16_t* At16 = ws.take<uint16_t>((size_t)E * in * RP);
+  float* gb = ws.take<float>((size_t)n_rows * r);
+  uint16_t* gb16 = ws.take<uint16_t>((size_t)n_rows * RP);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if ((rc = launch_pad(B, E, out, r, 1, Bt16, RP, out, st))) return rc;
+  if ((rc = launch_pad(A, E, r, in, 1, At16, in, RP, st))) return rc;
+  if ((rc = launch_moe_rowdot(g, nullptr, Bt16, expert_offsets, blk_prefix, n_rows, E, out, r, RP,
+                              scale, gb, gb16, st)))
+    return rc;
+  if ((rc = launch_moe_gemm(W_t, g, nullptr, At16, gb16, dx, expert_offsets, tile_prefix, n_rows, in,
+                            out, E, RP, st)))
+    return rc;
+  if ((rc = launch_moe_coldot(x, gather, gb, expert_offsets, E, in, r, scale, 1, dA, st))) return rc;
+  return launch_moe_coldot(g, nullptr, xa, expert_offsets, E, out, r, scale, 0, dB, st);
+}
+
+int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_t R, int64_t C,
+                                    artk_stream_t stream) {
+  ARTK_CHECK_ARG(in && out, "null pointer argument");
+  ARTK_CHECK_ARG(n > 0 && n < 65536 && R > 0 && C > 0, "n, R, C must be positive (n < 65536)");
+  dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)n);
+  transpose_bf16_batched_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)in,
+                                                                       (uint16_t*)out, R, C);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+}  // extern "C"

@@ -282,6 +282,101 @@ def lora_linear_bwd(g, x, W_t, A, B, xa, scale: float):
 
 
 # -----------------------------------------------------------------------------
+# MoE expert path
+# -----------------------------------------------------------------------------
+class Routing:
+    """Device tensors that describe one routing decision (see artk_moe_route)."""
+
+    __slots__ = ("topk_idx", "topk_w", "perm", "inv_perm", "row_token", "offsets", "tile_prefix",
+                 "blk_prefix", "n_rows", "n_experts", "k")
+
+
+def moe_route(router_logits: torch.Tensor, k: int) -> Routing:
+    T, E = router_logits.shape
+    _need(router_logits, "router_logits", torch.float32)
+    lib = _lib.load()
+    dev = router_logits.device
+    i32 = lambda *shape: torch.empty(shape, dtype=torch.int32, device=dev)
+    r = Routing()
+    r.topk_idx, r.topk_w = i32(T, k), torch.empty((T, k), dtype=torch.float32, device=dev)
+    r.perm, r.inv_perm, r.row_token = i32(T * k), i32(T * k), i32(T * k)
+    r.offsets, r.tile_prefix, r.blk_prefix = i32(E + 1), i32(E + 1), i32(E + 1)
+    r.n_rows, r.n_experts, r.k = T * k, E, k
+    ws = _workspace(lib.artk_moe_route_workspace_bytes(T, E, k), dev)
+    _lib.check(
+        lib.artk_moe_route(router_logits.data_ptr(), T, E, k, r.topk_idx.data_ptr(),
+                           r.topk_w.data_ptr(), r.perm.data_ptr(), r.inv_perm.data_ptr(),
+                           r.row_token.data_ptr(), r.offsets.data_ptr(), r.tile_prefix.data_ptr(),
+                           r.blk_prefix.data_ptr(), ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return r
+
+
+def transpose_batched(x: torch.Tensor) -> torch.Tensor:
+    """out[b, c, r] = x[b, r, c] for a contiguous bf16 [n, R, C] tensor."""
+    _need(x, "x", torch.bfloat16)
+    n, R, C = x.shape
+    out = torch.empty((n, C, R), dtype=torch.bfloat16, device=x.device)
+    _lib.check(_lib.load().artk_transpose_bf16_batched(x.data_ptr(), out.data_ptr(), n, R, C,
+                                                        _stream(x.device)))
+    return out
+
+
+def moe_lora_grouped_fwd(x, gather, W, A, B, scale: float, routing: Routing):
+    """(y bf16 [n_rows,out], xa f32 [n_rows,r]); x bf16 [*,in], W bf16 [E,out,in]."""
+    E, n_out, n_in = W.shape
+    r = A.shape[1]
+    _need(x, "x", torch.bfloat16)
+    _need(W, "W", torch.bfloat16)
+    _need(A, "A", torch.bfloat16, (E, r, n_in))
+    _need(B, "B", torch.bfloat16, (E, n_out, r))
+    if gather is not None:
+        _need(gather, "gather", torch.int32, (routing.n_rows,))
+    elif x.shape[0] != routing.n_rows:
+        raise ValueError("x must have one row per sorted (token, expert) pair when gather is None")
+    lib = _lib.load()
+    dev = x.device
+    n = routing.n_rows
+    y = torch.empty((n, n_out), dtype=torch.bfloat16, device=dev)
+    xa = torch.empty((n, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_moe_lora_grouped_fwd_workspace_bytes(n, n_in, n_out, E, r), dev)
+    _lib.check(
+        lib.artk_moe_lora_grouped_fwd(x.data_ptr(), _ptr(gather), W.data_ptr(), A.data_ptr(),
+                                      B.data_ptr(), scale, routing.offsets.data_ptr(),
+                                      routing.tile_prefix.data_ptr(), routing.blk_prefix.data_ptr(), n,
+                                      n_in, n_out, E, r, y.data_ptr(), xa.data_ptr(), ws.data_ptr(),
+                                      ws.numel(), _stream(dev))
+    )
+    return y, xa
+
+
+def moe_lora_grouped_bwd(g, x, gather, W_t, A, B, xa, scale: float, routing: Routing):
+    """(dx bf16 [n_rows,in], dA f32 [E,r,in], dB f32 [E,out,r])."""
+    E, n_in, n_out = W_t.shape
+    r = A.shape[1]
+    n = routing.n_rows
+    _need(g, "g", torch.bfloat16, (n, n_out))
+    _need(x, "x", torch.bfloat16)
+    _need(W_t, "W_t", torch.bfloat16)
+    _need(xa, "xa", torch.float32, (n, r))
+    lib = _lib.load()
+    dev = x.device
+    dx = torch.empty((n, n_in), dtype=torch.bfloat16, device=dev)
+    dA = torch.empty((E, r, n_in), dtype=torch.float32, device=dev)
+    dB = torch.empty((E, n_out, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_moe_lora_grouped_bwd_workspace_bytes(n, n_in, n_out, E, r), dev)
+    _lib.check(
+        lib.artk_moe_lora_grouped_bwd(g.data_ptr(), x.data_ptr(), _ptr(gather), W_t.data_ptr(),
+                                      A.data_ptr(), B.data_ptr(), xa.data_ptr(), scale,
+                                      routing.offsets.data_ptr(), routing.tile_prefix.data_ptr(),
+                                      routing.blk_prefix.data_ptr(), n, n_in, n_out, E, r,
+                                      dx.data_ptr(), dA.data_ptr(), dB.data_ptr(), ws.data_ptr(),
+                                      ws.numel(), _stream(dev))
+    )
+    return dx, dA, dB
+
+
+# -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------
 PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM = range(5)

@@ -38,7 +38,10 @@ def parse():
     ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4"])
     ap.add_argument("--chunk-tokens", type=int, default=0, help="positions per logits scratch chunk")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=512)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also run one plain device copy of this size (scales FETCH_SIZE/WRITE_SIZE "
+                         "counters when profiling with rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -107,6 +110,14 @@ def main():
     def step():
         ops.grpo_fused(hidden, lm_head, lm_head_t, tokens, old, adv, mask, weights, None, T, 0.8,
                        1.2, 0.0, chunk, workspace=ws, out=out)
+
+    if args.copy_calibration_mib:
+        n = args.copy_calibration_mib << 20
+        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

@@ -154,6 +154,58 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
                              size_t workspace_bytes, artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * A9 — MoE expert path (no counterpart in the reference at this commit; the
+ * contract is the benchmark configuration: 128 experts, top-8, rank-8 LoRA per
+ * expert, tokens permuted into expert-contiguous groups).
+ *
+ * artk_moe_route: top-k experts per token and the expert-contiguous permutation.
+ *   router_logits f32 [T,E]
+ *   topk_idx i32 [T,k]   experts by decreasing logit, ties to the lower index
+ *   topk_w   f32 [T,k]   softmax probabilities of the chosen experts, renormalised
+ *   perm     i32 [T*k]   perm[i] = flat (token*k + slot) index of sorted row i;
+ *                        stable sort of the token-major list by expert id
+ *   inv_perm i32 [T*k]   inverse of perm;  row_token i32 [T*k] = perm[i] / k
+ *   expert_offsets i32 [E+1]  first sorted row of each expert
+ *   tile_prefix, blk_prefix i32 [E+1]  work lists of the grouped kernels
+ *     (prefix sums of ceil(rows_e/256) and ceil(rows_e/16))
+ * ------------------------------------------------------------------------- */
+size_t artk_moe_route_workspace_bytes(int64_t T, int32_t E, int32_t k);
+int32_t artk_moe_route(const float* router_logits, int64_t T, int32_t E, int32_t k, int32_t* topk_idx,
+                       float* topk_w, int32_t* perm, int32_t* inv_perm, int32_t* row_token,
+                       int32_t* expert_offsets, int32_t* tile_prefix, int32_t* blk_prefix,
+                       void* workspace, size_t workspace_bytes, artk_stream_t stream);
+
+/* Per-expert LoRA linear over the sorted rows:
+ *   y[i,:] = x[src(i),:] W_e^T + scale (x[src(i),:] A_e^T) B_e^T,  e = expert of row i
+ *   src(i) = gather[i] when gather != NULL (rows of x picked by row_token), else i.
+ *   W bf16 [E,out,in], A bf16 [E,r,in], B bf16 [E,out,r]
+ *   y bf16 [n_rows,out] out, xa f32 [n_rows,r] out (kept for the backward) */
+size_t artk_moe_lora_grouped_fwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
+                                                 int32_t r);
+int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const void* W, const void* A,
+                                  const void* B, float scale, const int32_t* expert_offsets,
+                                  const int32_t* tile_prefix, const int32_t* blk_prefix,
+                                  int64_t n_rows, int64_t in, int64_t out, int32_t E, int32_t r,
+                                  void* y, float* xa, void* workspace, size_t workspace_bytes,
+                                  artk_stream_t stream);
+
+/* Backward of the above for g bf16 [n_rows,out]:
+ *   dx bf16 [n_rows,in] (per sorted row; the caller sums the k rows of a token)
+ *   dA f32 [E,r,in], dB f32 [E,out,r];  W_t bf16 [E,in,out] (artk_transpose_bf16_batched) */
+size_t artk_moe_lora_grouped_bwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
+                                                 int32_t r);
+int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* gather, const void* W_t,
+                                  const void* A, const void* B, const float* xa, float scale,
+                                  const int32_t* expert_offsets, const int32_t* tile_prefix,
+                                  const int32_t* blk_prefix, int64_t n_rows, int64_t in, int64_t out,
+                                  int32_t E, int32_t r, void* dx, float* dA, float* dB,
+                                  void* workspace, size_t workspace_bytes, artk_stream_t stream);
+
+/* out[b,c,r] = in[b,r,c] for n bf16 [R,C] matrices. */
+int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_t R, int64_t C,
+                                    artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
  * artk_profile_enable(1) makes later calls bracket each dominant kernel with
  * HIP events on the launch stream; after the caller has synchronised,
