@@ -35,7 +35,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe"],
+                    help="c3 (default, the headline): fused GRPO step at the Qwen2.5-7B shape; c1/c4: the "
+                         "0.5B / 14B shapes; lora: LoRA linear fwd+bwd at the Qwen2.5-3B shapes; moe: "
+                         "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
     ap.add_argument("--chunk-tokens", type=int, default=0, help="positions per logits scratch chunk")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
@@ -71,6 +74,171 @@ def cpu_baseline(case, sample_tokens: int):
     }
 
 
+def timed(fn, steps, warmup):
+    """Seconds per call: `warmup` untimed calls, then `steps` calls between device syncs."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def base_result(args, metric, unit, value, ms_per_step, workload):
+    return {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": {"workload": workload},
+    }
+
+
+def bench_lora(args):
+    """LoRA linear fwd+bwd over the six projections of one Qwen2.5-3B layer that have
+    in = 2048 (q, o: out 2048; k, v: out 256; gate, up: out 11008), T = 8192, r = 8, alpha = 16.
+    One step = forward + backward of all six; value = algorithmic TFLOP/s of the step."""
+    import math
+
+    import torch
+
+    from art_amd import ops
+
+    dev = torch.device("cuda:0")
+    T, n_in, r, scale = 8192, 2048, 8, 2.0
+    g = torch.Generator().manual_seed(1002)
+    x = torch.randn(T, n_in, generator=g).to(torch.bfloat16).to(dev)
+    shapes = []
+    for name, n_out in (("q", 2048), ("o", 2048), ("k", 256), ("v", 256), ("gate", 11008), ("up", 11008)):
+        W = (0.02 * torch.randn(n_out, n_in, generator=g)).to(torch.bfloat16).to(dev)
+        A = ((torch.rand(r, n_in, generator=g) * 2 - 1) / math.sqrt(n_in)).to(torch.bfloat16).to(dev)
+        B = (0.01 * torch.randn(n_out, r, generator=g)).to(torch.bfloat16).to(dev)
+        up = torch.randn(T, n_out, generator=g).to(torch.bfloat16).to(dev)
+        shapes.append((name, n_out, W, ops.transpose(W), A, B, up))
+    flops = lambda n_out: 4.0 * T * n_in * n_out + 6.0 * T * r * (n_in + n_out)
+
+    def one(sh):
+        _, _, W, Wt, A, B, up = sh
+        y, xa = ops.lora_linear_fwd(x, W, A, B, scale)
+        ops.lora_linear_bwd(up, x, Wt, A, B, xa, scale)
+
+    def step():
+        for sh in shapes:
+            one(sh)
+
+    per_shape = {}
+    for sh in shapes[::2]:
+        dt = timed(lambda: one(sh), args.steps, args.warmup)
+        per_shape[f"out={sh[1]}"] = {"us_fwd_bwd": dt * 1e6, "tflops": flops(sh[1]) / dt / 1e12,
+                                     "frac": flops(sh[1]) / dt / 1e12 / PEAK_BF16_TFLOPS}
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one(shapes[4])
+    torch.cuda.synchronize()
+    gemm_ms, gemm_n = ops.profile_collect(ops.PROF_LORA_GEMM)
+    ops.profile_enable(False)
+    dt = timed(step, args.steps, 0)
+    total = sum(flops(sh[1]) for sh in shapes)
+    res = base_result(args, "LoRA linear fwd+bwd TFLOP/s (Qwen2.5-3B shapes)", "TFLOP/s", total / dt / 1e12,
+                      dt * 1e3, "C2-lora-qwen2.5-3b")
+    res["config"].update({"tokens": T, "in": n_in, "rank": r, "projections": "q,o,k,v,gate,up"})
+    res["frac_of_bf16_peak"] = total / dt / 1e12 / PEAK_BF16_TFLOPS
+    res["shapes"] = per_shape
+    launch_ms = gemm_ms / max(gemm_n, 1)
+    ach = 2.0 * T * n_in * 11008 / (launch_ms * 1e-3) / 1e12
+    res["roofline"] = {"kernel": "lora_gemm_kernel (gate/up, fwd and dx launches)", "bound": "mfma",
+                       "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import lora_oracle
+
+        _, n_out, W, _, A, B, up = shapes[0]
+        t0 = time.perf_counter()
+        lora_oracle.lora_linear_grads(x.cpu(), W.cpu(), A.cpu(), B.cpu(), scale, up.cpu())
+        cdt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": flops(n_out) / cdt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"q projection (out=2048) fwd+bwd, fp32 torch-CPU oracle, 1 run of {cdt:.1f} s"}
+    print(json.dumps(res))
+
+
+def bench_moe(args):
+    """Expert-LoRA grouped GEMMs: 8192 tokens, hidden 2048, 128 experts, top-8, gate/up [768,2048],
+    down [2048,768], rank 8.  One step = routing + forward and backward of the three projections."""
+    import torch
+
+    from art_amd import ops
+
+    dev = torch.device("cuda:0")
+    T, H, I, E, k, r, scale = 8192, 2048, 768, 128, 8, 8, 2.0
+    g = torch.Generator().manual_seed(1005)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    logits = torch.randn(T, E, generator=g).to(dev)
+    mk = lambda o, i: ((0.02 * torch.randn(E, o, i, generator=g)).to(torch.bfloat16).to(dev),
+                       ((torch.rand(E, r, i, generator=g) * 2 - 1) / i ** 0.5).to(torch.bfloat16).to(dev),
+                       (0.01 * torch.randn(E, o, r, generator=g)).to(torch.bfloat16).to(dev))
+    Wg, Ag, Bg = mk(I, H)
+    Wu, Au, Bu = mk(I, H)
+    Wd, Ad, Bd = mk(H, I)
+    Wgt, Wut, Wdt = (ops.transpose_batched(w) for w in (Wg, Wu, Wd))
+    n = T * k
+    h = torch.randn(n, I, generator=g).to(torch.bfloat16).to(dev)
+    g_i = torch.randn(n, I, generator=g).to(torch.bfloat16).to(dev)
+    g_h = torch.randn(n, H, generator=g).to(torch.bfloat16).to(dev)
+
+    def step():
+        rt = ops.moe_route(logits, k)
+        yg, xag = ops.moe_lora_grouped_fwd(x, rt.row_token, Wg, Ag, Bg, scale, rt)
+        yu, xau = ops.moe_lora_grouped_fwd(x, rt.row_token, Wu, Au, Bu, scale, rt)
+        yd, xad = ops.moe_lora_grouped_fwd(h, None, Wd, Ad, Bd, scale, rt)
+        ops.moe_lora_grouped_bwd(g_h, h, None, Wdt, Ad, Bd, xad, scale, rt)
+        ops.moe_lora_grouped_bwd(g_i, x, rt.row_token, Wut, Au, Bu, xau, scale, rt)
+        ops.moe_lora_grouped_bwd(g_i, x, rt.row_token, Wgt, Ag, Bg, xag, scale, rt)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    gemm_ms, gemm_n = ops.profile_collect(ops.PROF_MOE_GEMM)
+    ops.profile_enable(False)
+    flops = 2 * (3 * 2.0 * n * H * I) + 3 * 6.0 * n * r * (H + I)  # fwd + dx of three projections + rank-r terms
+    res = base_result(args, "MoE expert-LoRA grouped GEMM fwd+bwd TFLOP/s", "TFLOP/s", flops / dt / 1e12, dt * 1e3,
+                      "C5-moe-qwen3-30b-a3b-share")
+    res["config"].update({"tokens": T, "hidden": H, "intermediate": I, "experts": E, "top_k": k, "rank": r})
+    res["frac_of_bf16_peak"] = flops / dt / 1e12 / PEAK_BF16_TFLOPS
+    launch_ms = gemm_ms / max(gemm_n, 1)
+    ach = 2.0 * n * H * I / (launch_ms * 1e-3) / 1e12
+    res["roofline"] = {"kernel": "moe_gemm_kernel (mean of the 6 launches per step)", "bound": "mfma",
+                       "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import moe_oracle
+
+        t0 = time.perf_counter()
+        ref = moe_oracle.route(logits.cpu(), k)
+        moe_oracle.grouped_lora_grads(x.cpu(), ref["row_token"], Wg.cpu(), Ag.cpu(), Bg.cpu(), scale,
+                                      ref["offsets"], g_i.cpu())
+        cdt = time.perf_counter() - t0
+        one = 2 * 2.0 * n * H * I + 6.0 * n * r * (H + I)
+        res["cpu_baseline"] = {"value": one / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"routing + gate projection fwd+bwd, fp32 torch-CPU oracle, 1 run of {cdt:.1f} s"}
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -85,6 +253,10 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.workload == "lora":
+        return bench_lora(args)
+    if args.workload == "moe":
+        return bench_moe(args)
     case = {"c1": synthetic.config1, "c3": synthetic.config3, "c4": synthetic.config4}[args.workload]()
     T, H = case.hidden.shape[1], case.hidden.shape[2]
     V = case.lm_head.shape[0]

@@ -34,7 +34,7 @@ def oracle_case(case, chunk):
                                      chunk_size=chunk)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 256), (260, 300, 128), (4, 1, 64),
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 768, 256), (264, 300, 128), (8, 1, 64),
                                    (1024, 512, 1024)])
 def test_gemm_nt_matches_fp32_matmul(artk_lib, gpu, M, N, K):
     print(f"gemm_nt M={M} N={N} K={K}", flush=True)
