@@ -1,38 +1,107 @@
-// Helpers shared by the LoRA linear and the MoE expert-LoRA kernels.
+// Helpers shared by the LoRA linear and the MoE expert-LoRA kernels: the rank-r
+// extra K steps of the GEMM epilogue and the skinny products.
 #pragma once
 #include "common.hpp"
+#include "gemm_nt.hpp"
 
 namespace artk {
 
-// dst [n][R1,C1] bf16 = zero-padded copy of src [n][R0,C0] (or of each matrix's
-// transpose).  One thread per destination element.
-__global__ __launch_bounds__(256) static void pad_copy_bf16_kernel(const uint16_t* __restrict__ src,
-                                                                   int64_t n, int64_t R0, int64_t C0,
-                                                                   int transpose,
-                                                                   uint16_t* __restrict__ dst,
-                                                                   int64_t R1, int64_t C1) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n * R1 * C1) return;
-  const int64_t b = i / (R1 * C1);
-  const int64_t j = i - b * R1 * C1;
-  const int64_t r = j / C1, c = j - r * C1;
-  const uint16_t* sp = src + b * R0 * C0;
-  uint16_t v = 0;
-  if (!transpose) {
-    if (r < R0 && c < C0) v = sp[r * C0 + c];
-  } else {
-    if (c < R0 && r < C0) v = sp[c * C0 + r];
-  }
-  dst[i] = v;
-}
-
 static inline int round16(int r) { return (r + 15) / 16 * 16; }
 
-static inline int32_t launch_pad(const void* src, int64_t n, int64_t R0, int64_t C0, int transpose,
-                                 uint16_t* dst, int64_t R1, int64_t C1, hipStream_t st) {
-  const int64_t total = n * R1 * C1;
-  pad_copy_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>((const uint16_t*)src, n, R0, C0,
-                                                                        transpose, dst, R1, C1);
+// acc += sum_e Qe[col, e] * Pe[row, e] for e < rp (rp a multiple of 16), as extra
+// K = 16 MFMA steps.  The operand fragments come straight from global memory in
+// MFMA layout: 16 bytes per lane = 8 consecutive e of row (lane % 32), first or
+// second half of the step by lane / 32.  Chunks at or past *_valid read as zero,
+// so a [rows, r] factor with r % 8 == 0 needs no padded copy.
+__device__ __forceinline__ void lowrank_steps(TileAcc& acc, const uint16_t* Pe, int pe_ld, int pe_valid,
+                                              const int64_t (&prow)[4], const uint16_t* Qe, int qe_ld,
+                                              int qe_valid, const int64_t (&qrow)[4], int rp) {
+  const int half = (threadIdx.x & 63) >> 5;
+  for (int e0 = 0; e0 < rp; e0 += 16) {
+    const int e = e0 + half * 8;
+    Frags f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+      f.p[i] = e < pe_valid ? *(const bf16x8*)(Pe + prow[i] * pe_ld + e) : z;
+      f.q[i] = e < qe_valid ? *(const bf16x8*)(Qe + qrow[i] * qe_ld + e) : z;
+    }
+    mma_frags(acc, f);
+  }
+}
+
+// Row products with MFMA 16x16x32: for the 16 rows held by the caller (lane % 16
+// selects the row behind xp / the factor row behind mp, lane / 16 the 8-element
+// K slice), accumulate over k = wave*32, wave*32 + 128, ...  Four independent
+// accumulators keep eight 16-byte loads in flight per lane.
+__device__ __forceinline__ floatx4 rowdot_accumulate(const uint16_t* xp, const uint16_t* mp,
+                                                     bool m_valid, int64_t K, int wave) {
+  floatx4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = a0, a2 = a0, a3 = a0;
+  const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  int64_t k = (int64_t)wave * 32;
+  for (; k + 384 < K; k += 512) {
+    const bf16x8 x0 = *(const bf16x8*)(xp + k), x1 = *(const bf16x8*)(xp + k + 128);
+    const bf16x8 x2 = *(const bf16x8*)(xp + k + 256), x3 = *(const bf16x8*)(xp + k + 384);
+    const bf16x8 m0 = m_valid ? *(const bf16x8*)(mp + k) : z;
+    const bf16x8 m1 = m_valid ? *(const bf16x8*)(mp + k + 128) : z;
+    const bf16x8 m2 = m_valid ? *(const bf16x8*)(mp + k + 256) : z;
+    const bf16x8 m3 = m_valid ? *(const bf16x8*)(mp + k + 384) : z;
+    a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x0, m0, a0, 0, 0, 0);
+    a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x1, m1, a1, 0, 0, 0);
+    a2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x2, m2, a2, 0, 0, 0);
+    a3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x3, m3, a3, 0, 0, 0);
+  }
+  for (; k < K; k += 128) {
+    const bf16x8 x0 = *(const bf16x8*)(xp + k);
+    const bf16x8 m0 = m_valid ? *(const bf16x8*)(mp + k) : z;
+    a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x0, m0, a0, 0, 0, 0);
+  }
+  return (a0 + a1) + (a2 + a3);
+}
+
+// Sum the four waves' accumulators (wave 0 ends up with the total).
+__device__ __forceinline__ floatx4 rowdot_block_sum(floatx4 acc, floatx4 (*red)[64]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave > 0) red[wave - 1][lane] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    acc += red[0][lane];
+    acc += red[1][lane];
+    acc += red[2][lane];
+  }
+  return acc;
+}
+
+// 4 bf16 -> 4 floats.
+__device__ __forceinline__ void unpack2(uint32_t w, float& lo, float& hi) {
+  lo = __uint_as_float(w << 16);
+  hi = __uint_as_float(w & 0xffff0000u);
+}
+
+// dst[c, r] = src[r, c] for small bf16 matrices; `which` selects one of two jobs so
+// that both transposes of a LoRA backward share a launch.
+struct SmallTranspose {
+  const uint16_t* src;
+  uint16_t* dst;
+  int64_t n, R, C;  // n matrices of [R, C]
+};
+__global__ __launch_bounds__(256) static void small_transpose2_kernel(SmallTranspose a, SmallTranspose b) {
+  const SmallTranspose t = blockIdx.y == 0 ? a : b;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= t.n * t.R * t.C) return;
+  const int64_t m = i / (t.R * t.C), j = i - m * t.R * t.C;
+  const int64_t c = j / t.R, r = j - c * t.R;  // dst index [c][r]
+  t.dst[i] = t.src[m * t.R * t.C + r * t.C + c];
+}
+
+static inline int32_t launch_small_transpose2(const void* s0, void* d0, int64_t n0, int64_t R0, int64_t C0,
+                                              const void* s1, void* d1, int64_t n1, int64_t R1, int64_t C1,
+                                              hipStream_t st) {
+  SmallTranspose a{(const uint16_t*)s0, (uint16_t*)d0, n0, R0, C0};
+  SmallTranspose b{(const uint16_t*)s1, (uint16_t*)d1, n1, R1, C1};
+  const int64_t big = n0 * R0 * C0 > n1 * R1 * C1 ? n0 * R0 * C0 : n1 * R1 * C1;
+  dim3 grid((unsigned)((big + 255) / 256), 2);
+  small_transpose2_kernel<<<grid, 256, 0, st>>>(a, b);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

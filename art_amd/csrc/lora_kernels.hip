@@ -9,10 +9,10 @@
 // are those packages' documented LoRA linear.
 //
 // The dense products run on the shared 256x256 MFMA main loop.  The rank-r
-// products ride along as extra K = 16 MFMA steps whose operands (the padded
-// low-rank factors) are read straight from global memory, so y and dx are each
-// one GEMM launch.  The skinny products (x A^T, g B: reductions along a row;
-// dA, dB: reductions along the token axis) are bandwidth-bound helpers.
+// products ride along as extra K = 16 MFMA steps whose operands (the low-rank
+// factors) are read straight from global memory, so y and dx are each one GEMM
+// launch.  The skinny products (x A^T, g B: reductions along a row; dA, dB:
+// reductions along the token axis) are bandwidth-bound helpers.
 #include "common.hpp"
 #include "gemm_nt.hpp"
 #include "lora_common.hpp"
@@ -23,13 +23,13 @@ namespace artk {
 // out[n, m] = sum_k Q[n,k] P[m,k] + sum_e Qe[n,e] Pe[m,e]     (bf16 out)
 // ----------------------------------------------------------------------------
 struct LoraGemmParams {
-  const void* P;    // [M,K] row operand (weight)
-  const void* Q;    // [N,K] column operand (activations)
-  const uint16_t* Pe;  // [M,RP] low-rank factor of the row operand, or nullptr
-  const uint16_t* Qe;  // [N,RP] low-rank factor of the column operand (scale folded in)
-  uint16_t* out;    // [N,M]
+  const void* P;       // [M,K] row operand (weight)
+  const void* Q;       // [N,K] column operand (activations)
+  const uint16_t* Pe;  // [M,r] low-rank factor of the row operand, or nullptr
+  const uint16_t* Qe;  // [N,RP] low-rank factor of the column operand (scale folded in, zero padded)
+  uint16_t* out;       // [N,M]
   int64_t M, N, K;
-  int RP, MT, NT;
+  int r, RP, MT, NT;
 };
 
 __global__ __launch_bounds__(NTHREADS) void lora_gemm_kernel(LoraGemmParams p) {
@@ -48,8 +48,6 @@ __global__ __launch_bounds__(NTHREADS) void lora_gemm_kernel(LoraGemmParams p) {
                (int)p.K);
 
   if (p.Pe != nullptr) {
-    // Rank-r part: operand fragments in MFMA layout come straight from global
-    // memory (16 bytes per lane: row = lane % 32, 8 consecutive e per half-wave).
     int64_t prow[4], qrow[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -58,15 +56,7 @@ __global__ __launch_bounds__(NTHREADS) void lora_gemm_kernel(LoraGemmParams p) {
       int64_t c = (int64_t)nt * TILE + wn * 128 + i * 32 + (lane & 31);
       qrow[i] = c < p.N ? c : p.N - 1;
     }
-    for (int e0 = 0; e0 < p.RP; e0 += 16) {
-      Frags f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        f.p[i] = *(const bf16x8*)(p.Pe + prow[i] * p.RP + e0 + half * 8);
-        f.q[i] = *(const bf16x8*)(p.Qe + qrow[i] * p.RP + e0 + half * 8);
-      }
-      mma_frags(acc, f);
-    }
+    lowrank_steps(acc, p.Pe, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
   }
 
 #pragma unroll
@@ -88,9 +78,9 @@ __global__ __launch_bounds__(NTHREADS) void lora_gemm_kernel(LoraGemmParams p) {
 }
 
 // ----------------------------------------------------------------------------
-// Row products: out[t, j] = sum_k X[t,k] Mt[j,k] for the 16 rows j0..j0+15 of
-// Mt (zero-padded factor, [RP,K]).  MFMA 16x16x32; a block owns 16 rows of X
-// and its 4 waves split K.  Writes f32 [T,R] (unscaled) and bf16 [T,RP] (scaled).
+// Row products: out[t, j] = sum_k X[t,k] Mt[j,k], Mt [R,K].  A block owns 16 rows
+// of X and 16 rows j0..j0+15 of Mt (rows >= R read as zero); its 4 waves split K.
+// Writes f32 [T,R] (unscaled) and bf16 [T,RP] (scaled, zero padded to RP).
 // ----------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restrict__ X,
                                                        const uint16_t* __restrict__ Mt, int64_t T,
@@ -104,106 +94,111 @@ __global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restric
   const int j0 = blockIdx.y * 16;
   int64_t trow = t0 + (lane & 15);
   if (trow >= T) trow = T - 1;
+  const int jm = j0 + (lane & 15);
   const uint16_t* xp = X + trow * K + (lane >> 4) * 8;
-  const uint16_t* mp = Mt + (int64_t)(j0 + (lane & 15)) * K + (lane >> 4) * 8;
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int64_t k = (int64_t)wave * 32; k < K; k += 128) {
-    bf16x8 a = *(const bf16x8*)(xp + k);
-    bf16x8 b = *(const bf16x8*)(mp + k);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
-  }
-  if (wave > 0) red[wave - 1][lane] = acc;
-  __syncthreads();
+  const uint16_t* mp = Mt + (int64_t)(jm < R ? jm : 0) * K + (lane >> 4) * 8;
+  floatx4 acc = rowdot_accumulate(xp, mp, jm < R, K, wave);
+  acc = rowdot_block_sum(acc, red);
   if (wave == 0) {
-    acc += red[0][lane];
-    acc += red[1][lane];
-    acc += red[2][lane];
     // lane holds column j = lane % 16 of rows (lane / 16) * 4 + e
-    const int j = j0 + (lane & 15);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int64_t t = t0 + (lane >> 4) * 4 + e;
       if (t < T) {
-        if (j < R) out_f32[t * R + j] = acc[e];
-        out_bf16[t * RP + j] = f32_to_bf16(acc[e] * scale);
+        if (jm < R) out_f32[t * R + jm] = acc[e];
+        out_bf16[t * RP + jm] = f32_to_bf16(acc[e] * scale);
       }
     }
   }
 }
 
 // ----------------------------------------------------------------------------
-// Column products over a slab of rows:
+// Column products over a slab of rows, two jobs per launch (dA and dB):
 //   partial[slab][c][r] = sum_{t in slab} X[t,c] Y[t,r]     r in [r0, r0+8)
-// X [T,C] bf16, Y [T,R] f32.  A thread owns 4 columns; Y rows are staged in LDS
+// X [T,C] bf16, Y [T,R] f32.  A thread owns 2 columns; Y rows are staged in LDS
 // and read as broadcasts.
 // ----------------------------------------------------------------------------
-constexpr int COLDOT_ROWS = 128;
+constexpr int COLDOT_MAX_ROWS = 256;
 
-__global__ __launch_bounds__(256) void coldot8_kernel(const uint16_t* __restrict__ X,
-                                                      const float* __restrict__ Y, int64_t T,
-                                                      int64_t C, int R, float* __restrict__ partial) {
-  __shared__ float ys[COLDOT_ROWS][8];
-  const int64_t c = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-  const int slab = blockIdx.y;
-  const int r0 = blockIdx.z * 8;
-  const int64_t t0 = (int64_t)slab * COLDOT_ROWS;
-  const int nrows = (int)((T - t0) < COLDOT_ROWS ? (T - t0) : COLDOT_ROWS);
-  for (int i = threadIdx.x; i < COLDOT_ROWS * 8; i += 256) {
+struct ColdotJob {
+  const uint16_t* X;
+  const float* Y;
+  float* partial;
+  float* out;
+  int64_t C;
+  int rows_per_slab, nslab, col_blocks, transpose_out;
+};
+
+__global__ __launch_bounds__(256) void coldot8_kernel(ColdotJob a, ColdotJob b, int64_t T, int R) {
+  __shared__ float ys[COLDOT_MAX_ROWS][8];
+  const int na = a.col_blocks * a.nslab;
+  const bool first = (int)blockIdx.x < na;
+  const ColdotJob j = first ? a : b;
+  const int bid = first ? blockIdx.x : blockIdx.x - na;
+  const int slab = bid / j.col_blocks, cb = bid - slab * j.col_blocks;
+  const int64_t c = ((int64_t)cb * 256 + threadIdx.x) * 2;
+  const int r0 = blockIdx.y * 8;
+  const int64_t t0 = (int64_t)slab * j.rows_per_slab;
+  const int nrows = (int)((T - t0) < j.rows_per_slab ? (T - t0) : j.rows_per_slab);
+  for (int i = threadIdx.x; i < j.rows_per_slab * 8; i += 256) {
     int rr = i >> 3, e = i & 7;
-    ys[rr][e] = rr < nrows ? Y[(t0 + rr) * R + r0 + e] : 0.f;
+    ys[rr][e] = rr < nrows ? j.Y[(t0 + rr) * R + r0 + e] : 0.f;
   }
   __syncthreads();
-  if (c >= C) return;
-  float acc[4][8];
+  if (c >= j.C) return;
+  float acc[2][8];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int q = 0; q < 2; ++q)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
-  const uint16_t* xp = X + t0 * C + c;
-#pragma unroll 4
+    for (int e = 0; e < 8; ++e) acc[q][e] = 0.f;
+  const uint16_t* xp = j.X + t0 * j.C + c;
+#pragma unroll 8
   for (int rr = 0; rr < nrows; ++rr) {
-    const uint2 raw = *(const uint2*)(xp + (int64_t)rr * C);
-    const float x0 = __uint_as_float(raw.x << 16), x1 = __uint_as_float(raw.x & 0xffff0000u);
-    const float x2 = __uint_as_float(raw.y << 16), x3 = __uint_as_float(raw.y & 0xffff0000u);
+    float x0, x1;
+    unpack2(*(const uint32_t*)(xp + (int64_t)rr * j.C), x0, x1);
     const floatx4 ya = *(const floatx4*)&ys[rr][0];
     const floatx4 yb = *(const floatx4*)&ys[rr][4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       acc[0][e] += x0 * ya[e];
       acc[1][e] += x1 * ya[e];
-      acc[2][e] += x2 * ya[e];
-      acc[3][e] += x3 * ya[e];
       acc[0][4 + e] += x0 * yb[e];
       acc[1][4 + e] += x1 * yb[e];
-      acc[2][4 + e] += x2 * yb[e];
-      acc[3][4 + e] += x3 * yb[e];
     }
   }
-  float* pp = partial + ((int64_t)slab * C + c) * R + r0;
+  float* pp = j.partial + ((int64_t)slab * j.C + c) * R + r0;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    *(floatx4*)(pp + (int64_t)j * R) = floatx4{acc[j][0], acc[j][1], acc[j][2], acc[j][3]};
-    *(floatx4*)(pp + (int64_t)j * R + 4) = floatx4{acc[j][4], acc[j][5], acc[j][6], acc[j][7]};
+  for (int q = 0; q < 2; ++q) {
+    *(floatx4*)(pp + (int64_t)q * R) = floatx4{acc[q][0], acc[q][1], acc[q][2], acc[q][3]};
+    *(floatx4*)(pp + (int64_t)q * R + 4) = floatx4{acc[q][4], acc[q][5], acc[q][6], acc[q][7]};
   }
 }
 
-// out = scale * sum over slabs; out is [C,R], or [R,C] when transpose_out.
-__global__ __launch_bounds__(256) void coldot_reduce_kernel(const float* __restrict__ partial,
-                                                            int nslab, int64_t C, int R, float scale,
-                                                            int transpose_out,
-                                                            float* __restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= C * R) return;
+// out = scale * sum over slabs (fixed order); out is [C,R], or [R,C] when
+// transpose_out.  64 outputs per block, 4 threads per output.
+__global__ __launch_bounds__(256) void coldot_reduce_kernel(ColdotJob a, ColdotJob b, int R, float scale) {
+  __shared__ float red[4][64];
+  const int nba = (int)((a.C * R + 63) / 64);
+  const bool first = (int)blockIdx.x < nba;
+  const ColdotJob j = first ? a : b;
+  const int bid = first ? blockIdx.x : blockIdx.x - nba;
+  const int64_t n = j.C * R;
+  const int64_t i = (int64_t)bid * 64 + (threadIdx.x & 63);
+  const int part = threadIdx.x >> 6;
   float s = 0.f;
-  for (int k = 0; k < nslab; ++k) s += partial[(int64_t)k * C * R + i];
-  s *= scale;
-  if (transpose_out) {
-    const int64_t c = i / R;
-    const int r = (int)(i - c * R);
-    out[(int64_t)r * C + c] = s;
-  } else {
-    out[i] = s;
+  if (i < n)
+    for (int k = part; k < j.nslab; k += 4) s += j.partial[(int64_t)k * n + i];
+  red[part][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (part == 0 && i < n) {
+    s = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x])) * scale;
+    if (j.transpose_out) {
+      const int64_t c = i / R;
+      const int r = (int)(i - c * R);
+      j.out[(int64_t)r * j.C + c] = s;
+    } else {
+      j.out[i] = s;
+    }
   }
 }
 
@@ -221,7 +216,8 @@ static int32_t check_lora(int64_t T, int64_t in, int64_t out, int r) {
 }
 
 static int32_t launch_lora_gemm(const void* P, const void* Q, const uint16_t* Pe, const uint16_t* Qe,
-                                void* out, int64_t M, int64_t N, int64_t K, int RP, hipStream_t st) {
+                                void* out, int64_t M, int64_t N, int64_t K, int r, int RP,
+                                hipStream_t st) {
   LoraGemmParams p;
   p.P = P;
   p.Q = Q;
@@ -231,6 +227,7 @@ static int32_t launch_lora_gemm(const void* P, const void* Q, const uint16_t* Pe
   p.M = M;
   p.N = N;
   p.K = K;
+  p.r = r;
   p.RP = RP;
   p.MT = (int)((M + TILE - 1) / TILE);
   p.NT = (int)((N + TILE - 1) / TILE);
@@ -242,30 +239,42 @@ static int32_t launch_lora_gemm(const void* P, const void* Q, const uint16_t* Pe
 }
 
 // out_f32 [T,R] = X Mt^T (unscaled), out_bf16 [T,RP] = scale * that, zero padded.
-static int32_t launch_rowdot(const void* X, const uint16_t* Mt_pad, int64_t T, int64_t K, int R,
-                             int RP, float scale, float* out_f32, uint16_t* out_bf16,
-                             hipStream_t st) {
+static int32_t launch_rowdot(const void* X, const void* Mt, int64_t T, int64_t K, int R, int RP,
+                             float scale, float* out_f32, uint16_t* out_bf16, hipStream_t st) {
   dim3 grid((unsigned)((T + 15) / 16), (unsigned)(RP / 16));
-  rowdot16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, Mt_pad, T, K, R, RP, scale, out_f32,
-                                        out_bf16);
+  rowdot16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, (const uint16_t*)Mt, T, K, R, RP, scale,
+                                        out_f32, out_bf16);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
 
-static int coldot_slabs(int64_t T) { return (int)((T + COLDOT_ROWS - 1) / COLDOT_ROWS); }
+// Slab height for a column product over T rows of a [T,C] matrix: enough blocks
+// to fill the chip without inflating the partial buffer.
+static int coldot_rows(int64_t T, int64_t C) {
+  const int64_t col_blocks = (C / 2 + 255) / 256;
+  for (int rows : {256, 128, 64})
+    if (col_blocks * ((T + rows - 1) / rows) >= 1024) return rows;
+  return 64;
+}
 
-// out = scale * X^T Y  ([C,R], or [R,C] when transpose_out); X [T,C] bf16, Y [T,R] f32.
-static int32_t launch_coldot(const void* X, const float* Y, int64_t T, int64_t C, int R, float scale,
-                             int transpose_out, float* partial, float* out, hipStream_t st) {
-  const int nslab = coldot_slabs(T);
-  dim3 grid((unsigned)((C / 4 + 255) / 256), (unsigned)nslab, (unsigned)(R / 8));
-  coldot8_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, Y, T, C, R, partial);
-  ARTK_CHECK_LAUNCH();
-  const int64_t n = C * R;
-  coldot_reduce_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(partial, nslab, C, R, scale,
-                                                                    transpose_out, out);
-  ARTK_CHECK_LAUNCH();
-  return ARTK_OK;
+static ColdotJob make_job(const void* X, const float* Y, float* partial, float* out, int64_t T,
+                          int64_t C, int transpose_out) {
+  ColdotJob j;
+  j.X = (const uint16_t*)X;
+  j.Y = Y;
+  j.partial = partial;
+  j.out = out;
+  j.C = C;
+  j.rows_per_slab = coldot_rows(T, C);
+  j.nslab = (int)((T + j.rows_per_slab - 1) / j.rows_per_slab);
+  j.col_blocks = (int)((C / 2 + 255) / 256);
+  j.transpose_out = transpose_out;
+  return j;
+}
+
+static size_t coldot_partial_floats(int64_t T, int64_t C, int R) {
+  const int rows = coldot_rows(T, C);
+  return (size_t)((T + rows - 1) / rows) * C * R;
 }
 
 }  // namespace artk
@@ -275,11 +284,10 @@ using namespace artk;
 extern "C" {
 
 size_t artk_lora_linear_fwd_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r) {
-  const int RP = round16(r);
+  (void)in;
+  (void)out;
   Workspace ws(nullptr, 0);
-  ws.take<uint16_t>((size_t)RP * in);   // A padded [RP,in]
-  ws.take<uint16_t>((size_t)out * RP);  // B padded [out,RP]
-  ws.take<uint16_t>((size_t)T * RP);    // s * x A^T, bf16 [T,RP]
+  ws.take<uint16_t>((size_t)T * round16(r));  // s * x A^T, bf16 [T,RP]
   return ws.used + 256;
 }
 
@@ -289,32 +297,29 @@ int32_t artk_lora_linear_fwd(const void* x, const void* W, const void* A, const 
   int32_t rc = check_lora(T, in, out, r);
   if (rc) return rc;
   ARTK_CHECK_ARG(x && W && A && B && y && xa, "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(y), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(A) && aligned16(B) && aligned16(y),
+                 "pointers must be 16-byte aligned");
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* A16 = ws.take<uint16_t>((size_t)RP * in);
-  uint16_t* B16 = ws.take<uint16_t>((size_t)out * RP);
   uint16_t* xa16 = ws.take<uint16_t>((size_t)T * RP);
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(A, 1, r, in, 0, A16, RP, in, st))) return rc;
-  if ((rc = launch_pad(B, 1, out, r, 0, B16, out, RP, st))) return rc;
-  if ((rc = launch_rowdot(x, A16, T, in, r, RP, scale, xa, xa16, st))) return rc;
-  return launch_lora_gemm(W, x, B16, xa16, y, out, T, in, RP, st);
+  if ((rc = launch_rowdot(x, A, T, in, r, RP, scale, xa, xa16, st))) return rc;
+  return launch_lora_gemm(W, x, (const uint16_t*)B, xa16, y, out, T, in, r, RP, st);
 }
 
 size_t artk_lora_linear_bwd_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r) {
   const int RP = round16(r);
   Workspace ws(nullptr, 0);
-  ws.take<uint16_t>((size_t)RP * out);  // B^T padded [RP,out]
-  ws.take<uint16_t>((size_t)in * RP);   // A^T padded [in,RP]
-  ws.take<float>((size_t)T * r);        // g B, f32 [T,r]
-  ws.take<uint16_t>((size_t)T * RP);    // s * g B, bf16 [T,RP]
-  const int64_t widest = in > out ? in : out;
-  ws.take<float>((size_t)coldot_slabs(T) * widest * r);
+  ws.take<uint16_t>((size_t)r * out);  // B^T [r,out]
+  ws.take<uint16_t>((size_t)in * r);   // A^T [in,r]
+  ws.take<float>((size_t)T * r);       // g B, f32 [T,r]
+  ws.take<uint16_t>((size_t)T * RP);   // s * g B, bf16 [T,RP]
+  ws.take<float>(coldot_partial_floats(T, in, r));
+  ws.take<float>(coldot_partial_floats(T, out, r));
   return ws.used + 256;
 }
 
@@ -329,26 +334,33 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
                  "pointers must be 16-byte aligned");
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* Bt16 = ws.take<uint16_t>((size_t)RP * out);
-  uint16_t* At16 = ws.take<uint16_t>((size_t)in * RP);
+  uint16_t* Bt = ws.take<uint16_t>((size_t)r * out);
+  uint16_t* At = ws.take<uint16_t>((size_t)in * r);
   float* gb = ws.take<float>((size_t)T * r);
   uint16_t* gb16 = ws.take<uint16_t>((size_t)T * RP);
-  const int64_t widest = in > out ? in : out;
-  float* partial = ws.take<float>((size_t)coldot_slabs(T) * widest * r);
+  float* part_a = ws.take<float>(coldot_partial_floats(T, in, r));
+  float* part_b = ws.take<float>(coldot_partial_floats(T, out, r));
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(B, 1, out, r, 1, Bt16, RP, out, st))) return rc;
-  if ((rc = launch_pad(A, 1, r, in, 1, At16, in, RP, st))) return rc;
-  // g B  -> gb (f32) and s * gb (bf16, padded)
-  if ((rc = launch_rowdot(g, Bt16, T, out, r, RP, scale, gb, gb16, st))) return rc;
+  // B^T [r,out] (factor of the g B row product) and A^T [in,r] (low-rank factor of dx)
+  if ((rc = launch_small_transpose2(B, Bt, 1, out, r, A, At, 1, r, in, st))) return rc;
+  if ((rc = launch_rowdot(g, Bt, T, out, r, RP, scale, gb, gb16, st))) return rc;
   // dx = g W + (s g B) A
-  if ((rc = launch_lora_gemm(W_t, g, At16, gb16, dx, in, T, out, RP, st))) return rc;
-  // dA [r,in] = s (g B)^T x ;  dB [out,r] = s g^T (x A^T)
-  if ((rc = launch_coldot(x, gb, T, in, r, scale, 1, partial, dA, st))) return rc;
-  return launch_coldot(g, xa, T, out, r, scale, 0, partial, dB, st);
+  if ((rc = launch_lora_gemm(W_t, g, At, gb16, dx, in, T, out, r, RP, st))) return rc;
+  // dA [r,in] = s (g B)^T x ;  dB [out,r] = s g^T (x A^T): one launch each for the
+  // slab products and the fixed-order reduction
+  ColdotJob ja = make_job(x, gb, part_a, dA, T, in, 1);
+  ColdotJob jb = make_job(g, xa, part_b, dB, T, out, 0);
+  dim3 grid((unsigned)(ja.col_blocks * ja.nslab + jb.col_blocks * jb.nslab), (unsigned)(r / 8));
+  coldot8_kernel<<<grid, 256, 0, st>>>(ja, jb, T, r);
+  ARTK_CHECK_LAUNCH();
+  const unsigned nred = (unsigned)((in * r + 63) / 64 + (out * r + 63) / 64);
+  coldot_reduce_kernel<<<nred, 256, 0, st>>>(ja, jb, r, scale);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
 }
 
 }  // extern "C"

@@ -167,13 +167,13 @@ struct MoeGemmParams {
   const void* W;           // [E,M,K] bf16
   const void* X;           // activations, [*,K] bf16
   const int* gather;       // permuted row i reads X row gather[i]; nullptr: row i
-  const uint16_t* Pe;      // [E,M,RP] padded low-rank factor of the weights
-  const uint16_t* Qe;      // [n_rows,RP] padded, scaled low-rank activations
+  const uint16_t* Pe;      // [E,M,r] low-rank factor of the weights
+  const uint16_t* Qe;      // [n_rows,RP] zero-padded, scaled low-rank activations
   uint16_t* out;           // [n_rows,M]
   const int* offsets;      // [E+1]
   const int* tile_prefix;  // [E+1]
   int64_t M, K;
-  int E, RP, MT;
+  int E, r, RP, MT;
 };
 
 __global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
@@ -198,7 +198,6 @@ __global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
                p.X, p.K, row0, row_end, 0, (int)p.K, p.gather);
 
   if (p.Pe != nullptr) {
-    const uint16_t* pe = p.Pe + (int64_t)e * p.M * p.RP;
     int64_t prow[4], qrow[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -207,15 +206,7 @@ __global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
       int c = wn * 128 + i * 32 + (lane & 31);
       qrow[i] = row0 + (c < nvalid ? c : nvalid - 1);
     }
-    for (int e0 = 0; e0 < p.RP; e0 += 16) {
-      Frags f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        f.p[i] = *(const bf16x8*)(pe + prow[i] * p.RP + e0 + half * 8);
-        f.q[i] = *(const bf16x8*)(p.Qe + qrow[i] * p.RP + e0 + half * 8);
-      }
-      mma_frags(acc, f);
-    }
+    lowrank_steps(acc, p.Pe + (int64_t)e * p.M * p.r, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
   }
 
 #pragma unroll
@@ -237,7 +228,7 @@ __global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
 }
 
 // Grouped row products: 16-row blocks never straddle experts.
-//   out[i, j] = sum_k X[row(i), k] Mt_e[j, k]
+//   out[i, j] = sum_k X[row(i), k] Mt_e[j, k],  Mt [E,R,K]
 __global__ __launch_bounds__(256) void moe_rowdot16_kernel(
     const uint16_t* __restrict__ X, const int* __restrict__ gather, const uint16_t* __restrict__ Mt,
     const int* __restrict__ offsets, const int* __restrict__ blk_prefix, int E, int64_t K, int R,
@@ -250,31 +241,21 @@ __global__ __launch_bounds__(256) void moe_rowdot16_kernel(
   const int64_t row_end = offsets[e + 1];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int j0 = blockIdx.y * 16;
+  const int jm = blockIdx.y * 16 + (lane & 15);
   int64_t row = row0 + (lane & 15);
   if (row >= row_end) row = row_end - 1;
   const int64_t src = gather ? gather[row] : row;
   const uint16_t* xp = X + src * K + (lane >> 4) * 8;
-  const uint16_t* mp = Mt + ((int64_t)e * RP + j0 + (lane & 15)) * K + (lane >> 4) * 8;
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t k = (int64_t)wave * 32; k < K; k += 128) {
-    bf16x8 a = *(const bf16x8*)(xp + k);
-    bf16x8 bb = *(const bf16x8*)(mp + k);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bb, acc, 0, 0, 0);
-  }
-  if (wave > 0) red[wave - 1][lane] = acc;
-  __syncthreads();
+  const uint16_t* mp = Mt + ((int64_t)e * R + (jm < R ? jm : 0)) * K + (lane >> 4) * 8;
+  floatx4 acc = rowdot_accumulate(xp, mp, jm < R, K, wave);
+  acc = rowdot_block_sum(acc, red);
   if (wave == 0) {
-    acc += red[0][lane];
-    acc += red[1][lane];
-    acc += red[2][lane];
-    const int j = j0 + (lane & 15);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int64_t i = row0 + (lane >> 4) * 4 + q;
       if (i < row_end) {
-        if (j < R) out_f32[i * R + j] = acc[q];
-        out_bf16[i * RP + j] = f32_to_bf16(acc[q] * scale);
+        if (jm < R) out_f32[i * R + jm] = acc[q];
+        out_bf16[i * RP + jm] = f32_to_bf16(acc[q] * scale);
       }
     }
   }
@@ -384,7 +365,7 @@ static int32_t check_moe(int64_t n_rows, int64_t in, int64_t out, int E, int r) 
 static int32_t launch_moe_gemm(const void* W, const void* X, const int* gather, const uint16_t* Pe,
                                const uint16_t* Qe, void* out, const int* offsets,
                                const int* tile_prefix, int64_t n_rows, int64_t M, int64_t K, int E,
-                               int RP, hipStream_t st) {
+                               int r, int RP, hipStream_t st) {
   MoeGemmParams p;
   p.W = W;
   p.X = X;
@@ -397,6 +378,7 @@ static int32_t launch_moe_gemm(const void* W, const void* X, const int* gather, 
   p.M = M;
   p.K = K;
   p.E = E;
+  p.r = r;
   p.RP = RP;
   p.MT = (int)((M + TILE - 1) / TILE);
   const int64_t max_row_tiles = (n_rows + TILE - 1) / TILE + E;
@@ -478,11 +460,11 @@ int32_t artk_moe_route(const float* router_logits, int64_t T, int32_t E, int32_t
 
 size_t artk_moe_lora_grouped_fwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
                                                  int32_t r) {
-  const int RP = round16(r);
+  (void)in;
+  (void)out;
+  (void)E;
   Workspace ws(nullptr, 0);
-  ws.take<uint16_t>((size_t)E * RP * in);
-  ws.take<uint16_t>((size_t)E * out * RP);
-  ws.take<uint16_t>((size_t)n_rows * RP);
+  ws.take<uint16_t>((size_t)n_rows * round16(r));
   return ws.used + 256;
 }
 
@@ -496,32 +478,29 @@ int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const vo
   if (rc) return rc;
   ARTK_CHECK_ARG(x && W && A && B && expert_offsets && tile_prefix && blk_prefix && y && xa,
                  "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(y), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(A) && aligned16(B) && aligned16(y),
+                 "pointers must be 16-byte aligned");
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* A16 = ws.take<uint16_t>((size_t)E * RP * in);
-  uint16_t* B16 = ws.take<uint16_t>((size_t)E * out * RP);
   uint16_t* xa16 = ws.take<uint16_t>((size_t)n_rows * RP);
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(A, E, r, in, 0, A16, RP, in, st))) return rc;
-  if ((rc = launch_pad(B, E, out, r, 0, B16, out, RP, st))) return rc;
-  if ((rc = launch_moe_rowdot(x, gather, A16, expert_offsets, blk_prefix, n_rows, E, in, r, RP, scale,
-                              xa, xa16, st)))
+  if ((rc = launch_moe_rowdot(x, gather, (const uint16_t*)A, expert_offsets, blk_prefix, n_rows, E, in,
+                              r, RP, scale, xa, xa16, st)))
     return rc;
-  return launch_moe_gemm(W, x, gather, B16, xa16, y, expert_offsets, tile_prefix, n_rows, out, in, E,
-                         RP, st);
+  return launch_moe_gemm(W, x, gather, (const uint16_t*)B, xa16, y, expert_offsets, tile_prefix, n_rows,
+                         out, in, E, r, RP, st);
 }
 
 size_t artk_moe_lora_grouped_bwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
                                                  int32_t r) {
   const int RP = round16(r);
   Workspace ws(nullptr, 0);
-  ws.take<uint16_t>((size_t)E * RP * out);
-  ws.take<uint16_t>((size_t)E * in * RP);
+  ws.take<uint16_t>((size_t)E * r * out);
+  ws.take<uint16_t>((size_t)E * in * r);
   ws.take<float>((size_t)n_rows * r);
   ws.take<uint16_t>((size_t)n_rows * RP);
   return ws.used + 256;
@@ -542,8 +521,8 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
                  "pointers must be 16-byte aligned");
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* Bt16 = ws.take<uint16_t>((size_t)E * RP * out);
-  uint16_t* At16 = ws.take<uint16_t>((size_t)E * in * RP);
+  uint16_t* Bt = ws.take<uint16_t>((size_t)E * r * out);  // [E,r,out]
+  uint16_t* At = ws.take<uint16_t>((size_t)E * in * r);   // [E,in,r]
   float* gb = ws.take<float>((size_t)n_rows * r);
   uint16_t* gb16 = ws.take<uint16_t>((size_t)n_rows * RP);
   if (!ws.ok()) {
@@ -551,13 +530,12 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_pad(B, E, out, r, 1, Bt16, RP, out, st))) return rc;
-  if ((rc = launch_pad(A, E, r, in, 1, At16, in, RP, st))) return rc;
-  if ((rc = launch_moe_rowdot(g, nullptr, Bt16, expert_offsets, blk_prefix, n_rows, E, out, r, RP,
-                              scale, gb, gb16, st)))
+  if ((rc = launch_small_transpose2(B, Bt, E, out, r, A, At, E, r, in, st))) return rc;
+  if ((rc = launch_moe_rowdot(g, nullptr, Bt, expert_offsets, blk_prefix, n_rows, E, out, r, RP, scale,
+                              gb, gb16, st)))
     return rc;
-  if ((rc = launch_moe_gemm(W_t, g, nullptr, At16, gb16, dx, expert_offsets, tile_prefix, n_rows, in,
-                            out, E, RP, st)))
+  if ((rc = launch_moe_gemm(W_t, g, nullptr, At, gb16, dx, expert_offsets, tile_prefix, n_rows, in, out,
+                            E, r, RP, st)))
     return rc;
   if ((rc = launch_moe_coldot(x, gather, gb, expert_offsets, E, in, r, scale, 1, dA, st))) return rc;
   return launch_moe_coldot(g, nullptr, xa, expert_offsets, E, out, r, scale, 0, dB, st);
