@@ -263,20 +263,24 @@ __global__ __launch_bounds__(256) void moe_rowdot16_kernel(
 
 // Grouped column products over the rows of one expert:
 //   out_e[c, r] = scale * sum_{i in rows(e)} X[row(i), c] Y[i, r]    r in [r0, r0+8)
-// out is [E,C,R], or [E,R,C] when transpose_out.  Fixed summation order.
+// out is [E,C,R], or [E,R,C] when transpose_out.  A block owns 128 columns of one
+// expert: 64 column pairs x 4 row groups (row group g takes rows g, g+4, ...),
+// merged through LDS in a fixed order.
 __global__ __launch_bounds__(256) void moe_coldot8_kernel(
     const uint16_t* __restrict__ X, const int* __restrict__ gather, const float* __restrict__ Y,
     const int* __restrict__ offsets, int64_t C, int R, float scale, int transpose_out,
     float* __restrict__ out) {
   __shared__ float ys[128][8];
   __shared__ int rows[128];
-  const int64_t c = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  __shared__ float red[3][64][17];
+  const int cp = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int64_t c = ((int64_t)blockIdx.x * 64 + cp) * 2;
   const int e = blockIdx.y;
   const int r0 = blockIdx.z * 8;
   const int64_t begin = offsets[e], end = offsets[e + 1];
-  float acc[4][8];
+  float acc[2][8];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int q = 0; q < 8; ++q) acc[j][q] = 0.f;
   for (int64_t s0 = begin; s0 < end; s0 += 128) {
@@ -288,37 +292,41 @@ __global__ __launch_bounds__(256) void moe_coldot8_kernel(
     }
     if (threadIdx.x < 128) {
       const int64_t i = s0 + threadIdx.x;
-      rows[threadIdx.x] = threadIdx.x < nrows ? (gather ? gather[i] : (int)i) : 0;
+      rows[threadIdx.x] = (int)threadIdx.x < nrows ? (gather ? gather[i] : (int)i) : 0;
     }
     __syncthreads();
     if (c < C) {
-      for (int rr = 0; rr < nrows; ++rr) {
-        const uint2 raw = *(const uint2*)(X + (int64_t)rows[rr] * C + c);
-        const float x0 = __uint_as_float(raw.x << 16), x1 = __uint_as_float(raw.x & 0xffff0000u);
-        const float x2 = __uint_as_float(raw.y << 16), x3 = __uint_as_float(raw.y & 0xffff0000u);
+#pragma unroll 4
+      for (int rr = rg; rr < nrows; rr += 4) {
+        float x0, x1;
+        unpack2(*(const uint32_t*)(X + (int64_t)rows[rr] * C + c), x0, x1);
         const floatx4 ya = *(const floatx4*)&ys[rr][0];
         const floatx4 yb = *(const floatx4*)&ys[rr][4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           acc[0][q] += x0 * ya[q];
           acc[1][q] += x1 * ya[q];
-          acc[2][q] += x2 * ya[q];
-          acc[3][q] += x3 * ya[q];
           acc[0][4 + q] += x0 * yb[q];
           acc[1][4 + q] += x1 * yb[q];
-          acc[2][4 + q] += x2 * yb[q];
-          acc[3][4 + q] += x3 * yb[q];
         }
       }
     }
   }
-  if (c >= C) return;
+  if (rg > 0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 8; ++q) red[rg - 1][cp][j * 8 + q] = acc[j][q];
+  }
+  __syncthreads();
+  if (rg != 0 || c >= C) return;
   float* oe = out + (int64_t)e * C * R;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      const float v = acc[j][q] * scale;
+      const float v =
+          (acc[j][q] + red[0][cp][j * 8 + q] + red[1][cp][j * 8 + q] + red[2][cp][j * 8 + q]) * scale;
       if (transpose_out)
         oe[(int64_t)(r0 + q) * C + c + j] = v;
       else
@@ -403,7 +411,7 @@ static int32_t launch_moe_rowdot(const void* X, const int* gather, const uint16_
 static int32_t launch_moe_coldot(const void* X, const int* gather, const float* Y, const int* offsets,
                                  int E, int64_t C, int R, float scale, int transpose_out, float* out,
                                  hipStream_t st) {
-  dim3 grid((unsigned)((C / 4 + 255) / 256), (unsigned)E, (unsigned)(R / 8));
+  dim3 grid((unsigned)((C / 2 + 63) / 64), (unsigned)E, (unsigned)(R / 8));
   moe_coldot8_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, gather, Y, offsets, C, R, scale,
                                            transpose_out, out);
   ARTK_CHECK_LAUNCH();
