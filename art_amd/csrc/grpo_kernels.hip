@@ -52,6 +52,60 @@ struct FwdParams {
   int VT, TT;
 };
 
+// Per-position (max, sum-exp) over this wave's 128 vocabulary rows and the gather
+// of the target logit.  RAGGED: the tile reaches past the last vocabulary row and
+// those rows are left out (last tile only).
+template <bool RAGGED>
+__device__ __forceinline__ void lse_epilogue(const TileAcc& acc, const FwdParams& p, int vt, int wm,
+                                             int64_t vbase, const int64_t (&y)[4],
+                                             const int (&col)[4]) {
+  const int lane = threadIdx.x & 63;
+  const int half = lane >> 5;
+  const int vleft = (int)(p.V - vbase < 128 ? p.V - vbase : 128);  // valid rows of this wave
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) {
+    // A position's 128 logits of this wave: 64 in this lane, 64 in lane^32.
+    float m = -INFINITY;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+        const float z = acc.c[mi][ni][j];
+        m = fmaxf(m, (RAGGED && r >= vleft) ? -INFINITY : z);
+      }
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    const float mb = (m == -INFINITY ? 0.f : m) * LOG2E;
+    float l = 0.f;
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][j], LOG2E, -mb));
+        l += (RAGGED && r >= vleft) ? 0.f : e;
+      }
+    l += __shfl_xor(l, 32, 64);
+    if (lane < 32 && col[ni] < p.Tc)
+      p.part[(int64_t)(vt * 2 + wm) * p.Tc + col[ni]] = make_float2(m, l);
+
+    // Gather: exactly one lane of one wave of the whole grid holds logit[y].
+    const int64_t rel = y[ni] - vbase;
+    const bool hit = rel >= 0 && rel < 128 && ((((int)rel) >> 2) & 1) == half;
+    if (__any(hit)) {
+      float s = 0.f;
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+          s = (r == (int)rel) ? acc.c[mi][ni][j] : s;
+        }
+      if (hit) p.sel[col[ni]] = s;
+    }
+  }
+}
+
 template <bool STASH>
 __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
@@ -102,55 +156,12 @@ __global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
     }
   }
 
-  // Vocab rows past V (last tile only) must not enter the reductions.
-  if ((int64_t)vt * TILE + TILE > p.V) {
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        int64_t v = vbase + mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
-        if (v >= p.V) {
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) acc.c[mi][ni][j] = -INFINITY;
-        }
-      }
-  }
-
-#pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    // A position's 128 logits of this wave: 64 in this lane, 64 in lane^32.
-    float m = -INFINITY;
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) m = fmaxf(m, acc.c[mi][ni][j]);
-    m = fmaxf(m, __shfl_xor(m, 32, 64));
-    const float mb = (m == -INFINITY ? 0.f : m) * LOG2E;
-    float l = 0.f;
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int j = 0; j < 16; ++j)
-        l += __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][j], LOG2E, -mb));
-    l += __shfl_xor(l, 32, 64);
-    if (lane < 32 && col[ni] < p.Tc)
-      p.part[(int64_t)(vt * 2 + wm) * p.Tc + col[ni]] = make_float2(m, l);
-
-    // Gather: exactly one lane of one wave of the whole grid holds logit[y].
-    const int64_t rel = y[ni] - vbase;
-    const bool hit = rel >= 0 && rel < 128 && ((((int)rel) >> 2) & 1) == half;
-    if (__any(hit)) {
-      float s = 0.f;
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
-          if (r == (int)rel) s = acc.c[mi][ni][j];
-        }
-      if (hit) p.sel[col[ni]] = s;
-    }
-  }
+  // The accumulators are only read from here on (writing to them would make the
+  // compiler shuttle all 256 between the accumulation and the vector registers).
+  if ((int64_t)vt * TILE + TILE > p.V)
+    lse_epilogue<true>(acc, p, vt, wm, vbase, y, col);
+  else
+    lse_epilogue<false>(acc, p, vt, wm, vbase, y, col);
 }
 
 // K2: merge the per-tile (max, sumexp) partials of each position.  A block

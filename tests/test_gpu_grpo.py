@@ -195,3 +195,82 @@ def test_config1_full_size(artk_lib, gpu):
     assert (logprob.cpu() - ref["logprobs"]).abs().max().item() <= LP_TOL
     assert abs(loss.item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item())
     assert rel_l2(hidden.grad.float().cpu(), ref["d_hidden"]) <= GRAD_TOL
+
+
+# ---------------------------------------------------------------------------------
+# Full-size configurations (BASELINE configs 3 and 4): the CPU oracle cannot run the
+# whole case in seconds, so parity is checked on windows of positions (every
+# position's logprob and d_hidden row depend on the rest of the batch only through
+# the scalar mask count) and through size-independent properties.
+# ---------------------------------------------------------------------------------
+def window_oracle(case, start, length, mask_count_full):
+    """Oracle logprobs and d_hidden rows for positions [start, start+length-1) of a
+    full-size case, evaluated on the window alone and rescaled to the batch's denominator."""
+    sl = slice(start, start + length)
+    cut = lambda t: t[:, sl].contiguous()
+    out = grpo_oracle.loss_and_grad(cut(case.hidden), case.lm_head, cut(case.tokens), cut(case.logprobs),
+                                    cut(case.advantages), cut(case.assistant_mask), cut(case.weights),
+                                    chunk_size=length)
+    m_win = grpo_oracle.shift_tensor(cut(case.assistant_mask), False).sum().item()
+    scale = (m_win + 1e-6) / (mask_count_full + 1e-6)
+    return out["logprobs"][0, :-1], out["d_hidden"][0, :-1] * scale
+
+
+def run_full_size(case, gpu, chunk_tokens):
+    T, H = case.hidden.shape[1], case.hidden.shape[2]
+    dev = case.to(gpu)
+    lm_head_t = ops.transpose(dev.lm_head)
+    new, _ = ops.logprob_fwd(dev.hidden.view(T, H), dev.lm_head, dev.tokens.view(T), True, T)
+    case.finish(new.cpu())
+    old = case.logprobs.view(T).to(gpu)
+    args = (dev.hidden.view(T, H), dev.lm_head, lm_head_t, dev.tokens.view(T), old, dev.advantages.view(T),
+            dev.assistant_mask.view(T), dev.weights.view(T), None, T, 0.8, 1.2, 0.0)
+    s, lp, dh = ops.grpo_fused(*args, chunk_tokens)
+    return args, s, lp, dh, new
+
+
+@pytest.mark.parametrize("name", ["c3", "c4"])
+def test_full_size_windows_and_properties(artk_lib, gpu, name):
+    print(f"full size {name}", flush=True)
+    case = synthetic.config3() if name == "c3" else synthetic.config4()
+    T, H = case.hidden.shape[1], case.hidden.shape[2]
+    args, s, lp, dh, new = run_full_size(case, gpu, 4096)
+    count = grpo_oracle.shift_tensor(case.assistant_mask, False).sum().item()
+    assert s[3].item() == count                       # integer mask count, bit-exact
+    assert torch.equal(lp, new)                        # fused forward == forward-only kernel
+    # windows: start of the row, a trajectory boundary, the end of the row
+    L = T // (32 if name == "c3" else 16)
+    for start in (0, 3 * L - 40, T - 96):
+        ref_lp, ref_dh = window_oracle(case, start, 96, count)
+        got_lp = lp[start:start + 95].cpu()
+        got_dh = dh[start:start + 95].float().cpu()
+        assert (got_lp - ref_lp).abs().max().item() <= LP_TOL
+        if ref_dh.abs().max().item() == 0.0:  # a window inside a zero-advantage group
+            assert got_dh.abs().max().item() == 0.0
+        else:
+            assert rel_l2(got_dh, ref_dh) <= GRAD_TOL
+    # rows with a zero coefficient (mask off, or zero advantage) are exactly zero
+    m = grpo_oracle.shift_tensor(case.assistant_mask, False)[0]
+    a = grpo_oracle.shift_tensor(case.advantages, 0.0)[0]
+    dead = (~m) | (a == 0)
+    assert dh[dead.to(gpu)].abs().max().item() == 0.0
+    # the remaining rows carry gradient unless the ratio was clipped (coefficient exactly 0)
+    nonzero = dh[(~dead).to(gpu)].float().abs().amax(dim=1) > 0
+    assert nonzero.float().mean().item() > 0.5
+    if name == "c4":
+        assert (a[m] == 0).any(), "config 4 must contain zero-variance groups"
+    # chunk-size invariance: forward bit-identical, loss and gradient within tolerance
+    s2, lp2, dh2 = ops.grpo_fused(*args, 2048)
+    assert torch.equal(lp2, lp)
+    assert abs(s2[0].item() - s[0].item()) <= 1e-6 * abs(s[0].item())
+    assert rel_l2(dh2.float(), dh.float()) <= 1e-3
+    # run-to-run determinism
+    s3, lp3, dh3 = ops.grpo_fused(*args, 4096)
+    assert torch.equal(s3, s) and torch.equal(dh3, dh)
+    # loss scalar against the oracle's loss body fed with the kernel's logprobs
+    loss_ref, _, _ = grpo_oracle.grpo_loss(
+        lp.cpu().view(1, T), grpo_oracle.shift_tensor(case.logprobs, 0.0),
+        grpo_oracle.shift_tensor(case.advantages, 0.0),
+        grpo_oracle.shift_tensor(case.assistant_mask, False).float(),
+        grpo_oracle.shift_tensor(case.weights, 0.0))
+    assert abs(s[0].item() - loss_ref.item()) <= LOSS_TOL * abs(loss_ref.item())
