@@ -7,9 +7,17 @@
 // matrix whose row index is the *contiguous* dimension of the output into the
 // P role, so that each lane owns 4 consecutive output elements.
 //
-// Work-group: 256 threads = 4 wavefronts (64 lanes) in a 2x2 grid, each
-// wavefront owns a 128x128 sub-tile = 4x4 MFMA 32x32x16 bf16 tiles, i.e. 256
-// fp32 accumulator registers per lane.  One work-group per CU (1 wave / SIMD).
+// Two work-group shapes share the code, selected by the template parameter NI
+// (column-operand MFMA tiles per wavefront):
+//   NI = 4: 256 threads = 4 wavefronts in a 2x2 grid, wave tile 128x128 = 4x4
+//           MFMA 32x32x16 tiles, 256 fp32 accumulators per lane, 1 wave / SIMD;
+//   NI = 2: 512 threads = 8 wavefronts in a 2x4 grid, wave tile 128x64 = 4x2
+//           tiles, 128 accumulators per lane, 2 waves / SIMD: while one wave
+//           waits (LDS data, a full texture-address FIFO, the barrier, its
+//           epilogue) the other keeps the MFMA pipe busy.
+// One work-group per CU either way (LDS bound).  Measured: NI = 2 is faster for
+// the long-K lm_head product with its heavy epilogue, NI = 4 for the short-K
+// LoRA / MoE products.
 //
 // Data path: HBM/L2 -> LDS by buffer_load_dwordx4 ... lds (no VGPR staging),
 // two LDS stages of 2 x 32 KiB, 16-byte chunks XOR-swizzled so that both the
@@ -28,7 +36,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 constexpr int TILE = 256;       // tile rows of either operand
 constexpr int BK = 64;          // K elements per LDS stage
-constexpr int NTHREADS = 256;   // 4 wavefronts
+template <int NI> constexpr int nthreads() { return 1024 / NI; }   // 256 or 512
 constexpr int OPER_STAGE_BYTES = TILE * BK * 2;          // 32 KiB
 constexpr int STAGE_BYTES = 2 * OPER_STAGE_BYTES;         // P + Q
 constexpr int NSTAGES = 2;
@@ -39,10 +47,13 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // Swizzle of the 16-byte chunk index within a 128-byte LDS row.
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-// One operand of the NT GEMM as seen by one wavefront's DMA instructions.
+// One operand of the NT GEMM as seen by one wavefront's DMA instructions
+// (2 * NI instructions of 1 KiB per wave and stage).
+template <int NI>
 struct OperandLoader {
+  static constexpr int DI = 2 * NI;
   __amdgpu_buffer_rsrc_t rsrc;
-  int voff[8];  // per-lane byte offset of the 8 DMA instructions of this wave
+  int voff[DI];  // per-lane byte offset of the DMA instructions of this wave
 
   // base: first element of the operand; ld: leading dimension in elements;
   // row0: first tile row; nrows: rows the operand really has (rows past the
@@ -58,8 +69,8 @@ struct OperandLoader {
     int nvalid = left >= TILE ? TILE : (int)left;
     int r = lane >> 3, pc = lane & 7;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int row = (wave * 8 + i) * 8 + r;
+    for (int i = 0; i < DI; ++i) {
+      int row = (wave * DI + i) * 8 + r;
       int kc = pc ^ swz(row);
       int64_t rc = row < nvalid ? row : nvalid - 1;
       if (gather) rc = gather[row0 + rc];
@@ -67,56 +78,62 @@ struct OperandLoader {
     }
   }
 
-  // Issue DMA instructions LO..HI-1 of this wave's 8 for K offset k0 (elements)
+  // Issue DMA instructions LO..HI-1 of this wave's DI for K offset k0 (elements)
   // into the 32 KiB operand stage at `stage` (LDS byte address, wave-uniform).
   template <int LO, int HI>
   __device__ __forceinline__ void issue(char* stage, int wave, int k0) const {
 #pragma unroll
     for (int i = LO; i < HI; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * 8 + i) * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * DI + i) * 1024), 16,
                                                voff[i], k0 * 2, 0, 0);
     }
   }
 };
 
+template <int NI>
 struct TileAcc {
-  floatx16 c[4][4];  // [mi][ni]
+  floatx16 c[4][NI];  // [mi][ni]
   __device__ __forceinline__ void zero() {
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
+      for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
         for (int j = 0; j < 16; ++j) c[mi][ni][j] = 0.f;
   }
 };
 
 // Row (P-operand index, tile-relative) of accumulator element j of MFMA tile mi
-// for this lane, and column (Q-operand index, tile-relative) of MFMA tile ni.
-__device__ __forceinline__ int acc_row(int wm, int mi, int j, int lane) {
-  return wm * 128 + mi * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-}
+// for this lane: wm * 128 + mi * 32 + (j / 4) * 8 + (lane / 32) * 4 + j % 4;
+// column (Q-operand index, tile-relative) of MFMA tile ni:
+template <int NI>
 __device__ __forceinline__ int acc_col(int wn, int ni, int lane) {
-  return wn * 128 + ni * 32 + (lane & 31);
+  return wn * (32 * NI) + ni * 32 + (lane & 31);
 }
+// Position of a wavefront in the 2 (row operand) x (8 / NI) (column operand) grid.
+template <int NI> __device__ __forceinline__ int wave_m(int wave) { return wave / (8 / NI); }
+template <int NI> __device__ __forceinline__ int wave_n(int wave) { return wave % (8 / NI); }
 
-// Operand fragments of one K=16 step: 4 row-operand and 4 column-operand reads.
+// Operand fragments of one K=16 step: 4 row-operand and NI column-operand reads.
+template <int NI>
 struct Frags {
-  bf16x8 p[4], q[4];
+  bf16x8 p[4], q[NI];
 };
 
-__device__ __forceinline__ void load_frags(Frags& f, const char* sp, const char* sq, int off) {
+template <int NI>
+__device__ __forceinline__ void load_frags(Frags<NI>& f, const char* sp, const char* sq, int off) {
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi) f.p[mi] = *(const bf16x8*)(sp + off + mi * 4096);
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) f.q[ni] = *(const bf16x8*)(sq + off + ni * 4096);
+  for (int ni = 0; ni < NI; ++ni) f.q[ni] = *(const bf16x8*)(sq + off + ni * 4096);
 }
 
-__device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
+template <int NI>
+__device__ __forceinline__ void mma_frags(TileAcc<NI>& acc, const Frags<NI>& f) {
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni)
+    for (int ni = 0; ni < NI; ++ni)
       acc.c[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.p[mi], f.q[ni], acc.c[mi][ni], 0, 0, 0);
 }
 
@@ -124,7 +141,7 @@ __device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
 // k_begin/k_end are multiples of BK, k_end > k_begin.  `smem` is GEMM_LDS_BYTES
 // of LDS, 1 KiB aligned.
 //
-// Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 16 MFMAs each):
+// Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 8 MFMAs each per wave):
 //   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read;
 //                the second half of the DMA for the next stage is issued here
 //   wait for own LDS reads and own DMA, barrier:
@@ -132,20 +149,20 @@ __device__ __forceinline__ void mma_frags(TileAcc& acc, const Frags& f) {
 //                current stage is free, and the next stage has landed
 //   step 3     : MFMAs while step 0 of the next stage is read; the first half
 //                of the DMA for the stage after next goes into the freed buffer
-// (the DMA issue is spread over 1.5 steps because the address FIFO of the
-// texture unit backs up and stalls the wave when 16 loads are issued at once)
 // The loop body has no branches: past the end, the DMA re-fetches the last
 // stage into the idle buffer and the fragment prefetch reads values nobody uses.
-__device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const void* P, int64_t ldp,
+template <int NI>
+__device__ __forceinline__ void gemm_tile_nt(TileAcc<NI>& acc, char* smem, const void* P, int64_t ldp,
                                              int64_t prow0, int64_t prows, const void* Q,
                                              int64_t ldq, int64_t qrow0, int64_t qrows, int k_begin,
                                              int k_end, const int* qgather = nullptr) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
+  constexpr int DI = 2 * NI;
 
-  OperandLoader lp, lq;
+  OperandLoader<NI> lp, lq;
   lp.init(P, ldp, prow0, prows, wave, lane);
   lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather);
 
@@ -158,22 +175,22 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
     for (int kk = 0; kk < 4; ++kk) off[kk] = rl * 128 + (((kk * 2 + (lane >> 5)) ^ f) << 4);
   }
   const int p_wave_off = wm * 128 * 128;
-  const int q_wave_off = OPER_STAGE_BYTES + wn * 128 * 128;
+  const int q_wave_off = OPER_STAGE_BYTES + wn * (32 * NI) * 128;
 
   const int nk = (k_end - k_begin) / BK;
   const int k_last = k_end - BK;
 
-  constexpr int EARLY = 4;  // DMA instructions per operand issued right after the barrier
-  lp.issue<0, 8>(smem, wave, k_begin);
-  lq.issue<0, 8>(smem + OPER_STAGE_BYTES, wave, k_begin);
+  constexpr int EARLY = NI;  // DMA instructions per operand issued right after the barrier
+  lp.template issue<0, DI>(smem, wave, k_begin);
+  lq.template issue<0, DI>(smem + OPER_STAGE_BYTES, wave, k_begin);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   {
     int k1 = k_begin + BK < k_last ? k_begin + BK : k_last;
-    lp.issue<0, EARLY>(smem + STAGE_BYTES, wave, k1);
-    lq.issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
+    lp.template issue<0, EARLY>(smem + STAGE_BYTES, wave, k1);
+    lq.template issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
   }
-  Frags f0, f1;
+  Frags<NI> f0, f1;
   load_frags(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
 
   for (int kt = 0; kt < nk; ++kt) {
@@ -185,8 +202,8 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
     {
       int k1 = k_begin + (kt + 1) * BK;
       k1 = k1 < k_last ? k1 : k_last;
-      lp.issue<EARLY, 8>(nxt, wave, k1);
-      lq.issue<EARLY, 8>(nxt + OPER_STAGE_BYTES, wave, k1);
+      lp.template issue<EARLY, DI>(nxt, wave, k1);
+      lq.template issue<EARLY, DI>(nxt + OPER_STAGE_BYTES, wave, k1);
     }
     load_frags(f1, sp, sq, off[1]);
     mma_frags(acc, f0);
@@ -194,16 +211,32 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
     mma_frags(acc, f1);
     load_frags(f1, sp, sq, off[3]);
     mma_frags(acc, f0);
+    // Interleave: 3 steps of 4*NI MFMAs, 3*(4+NI) LDS reads, 2*(DI-EARLY) DMA issues.
+    if constexpr (NI == 4) {
 #pragma unroll
-    for (int i = 0; i < 2 * (8 - EARLY); ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-    }
+      for (int i = 0; i < 2 * (DI - EARLY); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+      }
 #pragma unroll
-    for (int i = 0; i < 24 - 2 * (8 - EARLY); ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+      for (int i = 0; i < 24 - 2 * (DI - EARLY); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2 * (DI - EARLY); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+      }
+#pragma unroll
+      for (int i = 0; i < 18 - 2 * (DI - EARLY); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
     }
 
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -211,15 +244,26 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc& acc, char* smem, const voi
 
     int k2 = k_begin + (kt + 2) * BK;
     k2 = k2 < k_last ? k2 : k_last;
-    lp.issue<0, EARLY>(cur, wave, k2);
-    lq.issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
+    lp.template issue<0, EARLY>(cur, wave, k2);
+    lq.template issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
     load_frags(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
     mma_frags(acc, f1);
+    // 4*NI MFMA, 4+NI LDS reads, 2*EARLY DMA issues
+    if constexpr (NI == 4) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
-      if (i < EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // 2 DMA issues
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        if (i < EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 6; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     }
   }
   // Drain the redundant tail DMA before the caller reuses or releases LDS.

@@ -13,6 +13,11 @@
 
 namespace artk {
 
+// Work-group shape of each GEMM kernel (see gemm_nt.hpp).
+constexpr int FWD_NI = 2;   // lm_head projection + log-sum-exp epilogue: 8 waves
+constexpr int BWD_NI = 2;   // d_hidden GEMM
+constexpr int GEMM_NI = 4;  // plain GEMM
+
 // ----------------------------------------------------------------------------
 // index helpers
 // ----------------------------------------------------------------------------
@@ -56,14 +61,14 @@ struct FwdParams {
 // of the target logit.  RAGGED: the tile reaches past the last vocabulary row and
 // those rows are left out (last tile only).
 template <bool RAGGED>
-__device__ __forceinline__ void lse_epilogue(const TileAcc& acc, const FwdParams& p, int vt, int wm,
-                                             int64_t vbase, const int64_t (&y)[4],
-                                             const int (&col)[4]) {
+__device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt, int wm,
+                                             int64_t vbase, const int64_t (&y)[FWD_NI],
+                                             const int (&col)[FWD_NI]) {
   const int lane = threadIdx.x & 63;
   const int half = lane >> 5;
   const int vleft = (int)(p.V - vbase < 128 ? p.V - vbase : 128);  // valid rows of this wave
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
+  for (int ni = 0; ni < FWD_NI; ++ni) {
     // A position's 128 logits of this wave: 64 in this lane, 64 in lane^32.
     float m = -INFINITY;
 #pragma unroll
@@ -107,35 +112,35 @@ __device__ __forceinline__ void lse_epilogue(const TileAcc& acc, const FwdParams
 }
 
 template <bool STASH>
-__global__ __launch_bounds__(NTHREADS) void lmhead_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   int vt, tt;
   tile_coords(id, p.VT, p.TT, vt, tt);
 
-  TileAcc acc;
+  TileAcc<FWD_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE,
                p.Tc, 0, (int)p.H);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<FWD_NI>(wave), wn = wave_n<FWD_NI>(wave);
   const int half = lane >> 5;
   const int64_t vbase = (int64_t)vt * TILE + wm * 128;  // first vocab row of this wave
 
   // Targets of this lane's 4 positions (issued early: consumed after the reductions).
-  int64_t y[4];
-  int col[4];
+  int64_t y[FWD_NI];
+  int col[FWD_NI];
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    col[ni] = tt * TILE + acc_col(wn, ni, lane);
+  for (int ni = 0; ni < FWD_NI; ++ni) {
+    col[ni] = tt * TILE + acc_col<FWD_NI>(wn, ni, lane);
     y[ni] = col[ni] < p.Tc ? target_id(p.ids, p.t0 + col[ni], p.S, p.shift) : (int64_t)-1;
   }
 
   if (STASH) {
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
+    for (int ni = 0; ni < FWD_NI; ++ni) {
       const bool want = col[ni] < p.Tc && p.need[col[ni]] != 0;
       if (!__any(want)) continue;
       if (want) {
@@ -468,7 +473,7 @@ struct BwdParams {
 
 // The grid is sized for the worst case (every row active); the work-groups
 // beyond the device-side schedule exit at once.
-__global__ __launch_bounds__(NTHREADS) void dhidden_gemm_kernel(BwdParams p) {
+__global__ __launch_bounds__(nthreads<BWD_NI>()) void dhidden_gemm_kernel(BwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int n_active = p.sched[0], TT = p.sched[1], nsplit = p.sched[2], n_work = p.sched[3];
   if ((int)blockIdx.x >= n_work) return;
@@ -482,19 +487,19 @@ __global__ __launch_bounds__(NTHREADS) void dhidden_gemm_kernel(BwdParams p) {
   const int kb = (int)((int64_t)split * KT / nsplit);
   const int ke = (int)((int64_t)(split + 1) * KT / nsplit);
 
-  TileAcc acc;
+  TileAcc<BWD_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.Wt, p.V, (int64_t)ht * TILE, p.H, p.P, p.V, (int64_t)tt * TILE,
                n_active, kb * BK, ke * BK, p.active_idx);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<BWD_NI>(wave), wn = wave_n<BWD_NI>(wave);
   const int half = lane >> 5;
   const int64_t rows_per_split = (int64_t)TT * TILE;
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    const int col = tt * TILE + acc_col(wn, ni, lane);  // compact row
+  for (int ni = 0; ni < BWD_NI; ++ni) {
+    const int col = tt * TILE + acc_col<BWD_NI>(wn, ni, lane);  // compact row
     if (col >= n_active) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -562,22 +567,22 @@ struct GemmParams {
   int MT, NT, out_f32;
 };
 
-__global__ __launch_bounds__(NTHREADS) void gemm_nt_kernel(GemmParams p) {
+__global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   int mt, nt;
   tile_coords(id, p.MT, p.NT, mt, nt);
-  TileAcc acc;
+  TileAcc<GEMM_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
                (int)p.K);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<GEMM_NI>(wave), wn = wave_n<GEMM_NI>(wave);
   const int half = lane >> 5;
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    const int64_t col = (int64_t)nt * TILE + acc_col(wn, ni, lane);
+  for (int ni = 0; ni < GEMM_NI; ++ni) {
+    const int64_t col = (int64_t)nt * TILE + acc_col<GEMM_NI>(wn, ni, lane);
     if (col >= p.N) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -685,9 +690,9 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   const unsigned grid = (unsigned)(p.VT * p.TT);
   prof_begin(PROF_LMHEAD_FWD, st);
   if (stash)
-    lmhead_fwd_kernel<true><<<grid, NTHREADS, 0, st>>>(p);
+    lmhead_fwd_kernel<true><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
   else
-    lmhead_fwd_kernel<false><<<grid, NTHREADS, 0, st>>>(p);
+    lmhead_fwd_kernel<false><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
   prof_end(PROF_LMHEAD_FWD, st);
   ARTK_CHECK_LAUNCH();
   lse_finalize_kernel<<<(unsigned)((Tc + 15) / 16), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
@@ -740,7 +745,7 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   const int64_t dense_cap = (int64_t)HT * TT * 16;
   const unsigned grid = (unsigned)(max_blocks < dense_cap ? max_blocks : dense_cap);
   prof_begin(PROF_DHIDDEN_GEMM, st);
-  dhidden_gemm_kernel<<<grid, NTHREADS, 0, st>>>(b);
+  dhidden_gemm_kernel<<<grid, nthreads<BWD_NI>(), 0, st>>>(b);
   prof_end(PROF_DHIDDEN_GEMM, st);
   ARTK_CHECK_LAUNCH();
   const int64_t n4 = Tc * H / 4;
@@ -1026,7 +1031,7 @@ int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t
   p.MT = (int)((M + TILE - 1) / TILE);
   p.NT = (int)((N + TILE - 1) / TILE);
   p.out_f32 = out_f32;
-  gemm_nt_kernel<<<(unsigned)(p.MT * p.NT), NTHREADS, 0, (hipStream_t)stream>>>(p);
+  gemm_nt_kernel<<<(unsigned)(p.MT * p.NT), nthreads<GEMM_NI>(), 0, (hipStream_t)stream>>>(p);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

@@ -13,19 +13,19 @@ static inline int round16(int r) { return (r + 15) / 16 * 16; }
 // MFMA layout: 16 bytes per lane = 8 consecutive e of row (lane % 32), first or
 // second half of the step by lane / 32.  Chunks at or past *_valid read as zero,
 // so a [rows, r] factor with r % 8 == 0 needs no padded copy.
-__device__ __forceinline__ void lowrank_steps(TileAcc& acc, const uint16_t* Pe, int pe_ld, int pe_valid,
+template <int NI>
+__device__ __forceinline__ void lowrank_steps(TileAcc<NI>& acc, const uint16_t* Pe, int pe_ld, int pe_valid,
                                               const int64_t (&prow)[4], const uint16_t* Qe, int qe_ld,
-                                              int qe_valid, const int64_t (&qrow)[4], int rp) {
+                                              int qe_valid, const int64_t (&qrow)[NI], int rp) {
   const int half = (threadIdx.x & 63) >> 5;
   for (int e0 = 0; e0 < rp; e0 += 16) {
     const int e = e0 + half * 8;
-    Frags f;
+    Frags<NI> f;
+    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-      f.p[i] = e < pe_valid ? *(const bf16x8*)(Pe + prow[i] * pe_ld + e) : z;
-      f.q[i] = e < qe_valid ? *(const bf16x8*)(Qe + qrow[i] * qe_ld + e) : z;
-    }
+    for (int i = 0; i < 4; ++i) f.p[i] = e < pe_valid ? *(const bf16x8*)(Pe + prow[i] * pe_ld + e) : z;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) f.q[i] = e < qe_valid ? *(const bf16x8*)(Qe + qrow[i] * qe_ld + e) : z;
     mma_frags(acc, f);
   }
 }

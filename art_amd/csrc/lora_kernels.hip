@@ -19,6 +19,8 @@
 
 namespace artk {
 
+constexpr int LORA_NI = 4;  // work-group shape of the LoRA GEMMs (see gemm_nt.hpp)
+
 // ----------------------------------------------------------------------------
 // out[n, m] = sum_k Q[n,k] P[m,k] + sum_e Qe[n,e] Pe[m,e]     (bf16 out)
 // ----------------------------------------------------------------------------
@@ -32,36 +34,39 @@ struct LoraGemmParams {
   int r, RP, MT, NT;
 };
 
-__global__ __launch_bounds__(NTHREADS) void lora_gemm_kernel(LoraGemmParams p) {
+__global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   int mt, nt;
   tile_coords(id, p.MT, p.NT, mt, nt);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<LORA_NI>(wave), wn = wave_n<LORA_NI>(wave);
   const int half = lane >> 5;
 
-  TileAcc acc;
+  TileAcc<LORA_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
                (int)p.K);
 
   if (p.Pe != nullptr) {
-    int64_t prow[4], qrow[4];
+    int64_t prow[4], qrow[LORA_NI];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
       prow[i] = r < p.M ? r : p.M - 1;
-      int64_t c = (int64_t)nt * TILE + wn * 128 + i * 32 + (lane & 31);
+    }
+#pragma unroll
+    for (int i = 0; i < LORA_NI; ++i) {
+      int64_t c = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, i, lane);
       qrow[i] = c < p.N ? c : p.N - 1;
     }
     lowrank_steps(acc, p.Pe, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
   }
 
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    const int64_t col = (int64_t)nt * TILE + acc_col(wn, ni, lane);
+  for (int ni = 0; ni < LORA_NI; ++ni) {
+    const int64_t col = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, ni, lane);
     if (col >= p.N) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -232,7 +237,7 @@ static int32_t launch_lora_gemm(const void* P, const void* Q, const uint16_t* Pe
   p.MT = (int)((M + TILE - 1) / TILE);
   p.NT = (int)((N + TILE - 1) / TILE);
   prof_begin(PROF_LORA_GEMM, st);
-  lora_gemm_kernel<<<(unsigned)(p.MT * p.NT), NTHREADS, 0, st>>>(p);
+  lora_gemm_kernel<<<(unsigned)(p.MT * p.NT), nthreads<LORA_NI>(), 0, st>>>(p);
   prof_end(PROF_LORA_GEMM, st);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;

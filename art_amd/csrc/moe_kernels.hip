@@ -21,6 +21,7 @@ namespace artk {
 // ----------------------------------------------------------------------------
 // Routing: one wavefront per token.
 // ----------------------------------------------------------------------------
+constexpr int MOE_NI = 4;  // work-group shape of the grouped GEMMs (see gemm_nt.hpp)
 constexpr int MOE_MAX_E = 256;
 constexpr int MOE_MAX_K = 16;
 
@@ -176,7 +177,7 @@ struct MoeGemmParams {
   int E, r, RP, MT;
 };
 
-__global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
+__global__ __launch_bounds__(nthreads<MOE_NI>()) void moe_gemm_kernel(MoeGemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int n_work = p.tile_prefix[p.E] * p.MT;
   if ((int)blockIdx.x >= n_work) return;
@@ -189,29 +190,32 @@ __global__ __launch_bounds__(NTHREADS) void moe_gemm_kernel(MoeGemmParams p) {
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave_m<MOE_NI>(wave), wn = wave_n<MOE_NI>(wave);
   const int half = lane >> 5;
 
-  TileAcc acc;
+  TileAcc<MOE_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, (const char*)p.W + (int64_t)e * p.M * p.K * 2, p.K, (int64_t)mt * TILE, p.M,
                p.X, p.K, row0, row_end, 0, (int)p.K, p.gather);
 
   if (p.Pe != nullptr) {
-    int64_t prow[4], qrow[4];
+    int64_t prow[4], qrow[MOE_NI];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
       prow[i] = r < p.M ? r : p.M - 1;
-      int c = wn * 128 + i * 32 + (lane & 31);
+    }
+#pragma unroll
+    for (int i = 0; i < MOE_NI; ++i) {
+      int c = acc_col<MOE_NI>(wn, i, lane);
       qrow[i] = row0 + (c < nvalid ? c : nvalid - 1);
     }
     lowrank_steps(acc, p.Pe + (int64_t)e * p.M * p.r, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
   }
 
 #pragma unroll
-  for (int ni = 0; ni < 4; ++ni) {
-    const int c = acc_col(wn, ni, lane);
+  for (int ni = 0; ni < MOE_NI; ++ni) {
+    const int c = acc_col<MOE_NI>(wn, ni, lane);
     if (c >= nvalid) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -391,7 +395,7 @@ static int32_t launch_moe_gemm(const void* W, const void* X, const int* gather, 
   p.MT = (int)((M + TILE - 1) / TILE);
   const int64_t max_row_tiles = (n_rows + TILE - 1) / TILE + E;
   prof_begin(PROF_MOE_GEMM, st);
-  moe_gemm_kernel<<<(unsigned)(max_row_tiles * p.MT), NTHREADS, 0, st>>>(p);
+  moe_gemm_kernel<<<(unsigned)(max_row_tiles * p.MT), nthreads<MOE_NI>(), 0, st>>>(p);
   prof_end(PROF_MOE_GEMM, st);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
