@@ -825,12 +825,18 @@ static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bo
   }
 }
 
-// Chunk length: the caller's wish, at most T, and small enough that a row
-// offset inside the logits scratch fits the 31-bit offsets of the GEMM loader.
+// Chunk length: the caller's wish (<= 0: automatic, about 6000 positions split
+// evenly), at most T, and small enough that a row offset inside the logits
+// scratch fits the 31-bit offsets of the GEMM loader.
 static int64_t clamp_chunk(int64_t T, int64_t V, int64_t chunk_tokens) {
-  if (chunk_tokens <= 0) chunk_tokens = 4096;
-  const int64_t cap = ((1ll << 30) - 1) / V / TILE * TILE;  // Tc * V * 2 bytes < 2^31
-  if (chunk_tokens > cap) chunk_tokens = cap > TILE ? cap : TILE;
+  int64_t cap = ((1ll << 30) - 1) / V / TILE * TILE;  // Tc * V * 2 bytes < 2^31
+  if (cap < TILE) cap = TILE;
+  if (chunk_tokens <= 0) {
+    const int64_t want = cap < 6144 ? cap : 6144;
+    const int64_t n = (T + want - 1) / want;
+    chunk_tokens = ((T + n - 1) / n + TILE - 1) / TILE * TILE;
+  }
+  if (chunk_tokens > cap) chunk_tokens = cap;
   if (chunk_tokens > T) chunk_tokens = T;
   return chunk_tokens;
 }

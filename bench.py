@@ -41,7 +41,7 @@ def parse():
                          "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
     ap.add_argument("--chunk-tokens", type=int, default=0, help="positions per logits scratch chunk")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this size (scales FETCH_SIZE/WRITE_SIZE "
                          "counters when profiling with rocprofv3 --pmc)")
@@ -273,7 +273,7 @@ def main():
     weights = case.weights.view(T).to(dev)
     lm_head_t = ops.transpose(lm_head)
 
-    chunk = args.chunk_tokens or ops.DEFAULT_CHUNK_TOKENS
+    chunk = args.chunk_tokens or ops.DEFAULT_CHUNK_TOKENS  # 0 = library default
     ws = torch.empty(ops.grpo_fused_workspace_bytes(T, V, H, chunk), dtype=torch.uint8, device=dev)
     out = (torch.empty(4, dtype=torch.float32, device=dev),
            torch.empty(T, dtype=torch.float32, device=dev),
@@ -314,6 +314,7 @@ def main():
     # dominant kernel: one launch covers `chunk` positions against the whole vocabulary
     fwd_launch_ms = fwd_ms / max(fwd_n, 1)
     launches_per_step = fwd_n / args.steps
+    chunk = chunk or -(-T // int(launches_per_step))  # report the chunk the library chose (approximate)
     flops_per_launch = 2.0 * T * V * H / launches_per_step
     achieved = flops_per_launch / (fwd_launch_ms * 1e-3) / 1e12
     bwd_launch_ms = bwd_ms / max(bwd_n, 1)
