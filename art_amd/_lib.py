@@ -36,8 +36,8 @@ SIGNATURES = {
     "artk_grpo_fused_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "artk_grpo_fused": (
         _i32,
-        [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _i64, _p, _p,
-         _p, _p, _sz, _p],
+        [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _i64, _i32, _p,
+         _p, _p, _p, _sz, _p],
     ),
     "artk_transpose_bf16": (_i32, [_p, _p, _i64, _i64, _p]),
     "artk_gemm_nt": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),

@@ -39,21 +39,43 @@ __device__ __forceinline__ int64_t target_id(const int64_t* ids, int64_t t, int6
   return shifted_index(t, S, shift, src) ? ids[src] : (int64_t)0;  // pad id 0 (train.py:79)
 }
 
+// The rows of one chunk.  Dense mode: row r is position t0 + r and there are
+// `cap` of them.  Compact mode (the forward is evaluated only for positions that
+// can contribute to the loss): row r is position row_token[r] and the number of
+// rows is min(cap, *n_all - c0), known only on the device; kernels are launched
+// for `cap` rows and the surplus work-groups / threads exit at once.
+struct ChunkRows {
+  const int* row_token;  // nullptr in dense mode; else already offset to the chunk's first row
+  const int* n_all;      // compact mode: number of compact rows of the whole batch
+  int64_t t0;
+  int c0, cap;
+  __device__ __forceinline__ int n() const {
+    if (n_all == nullptr) return cap;
+    int left = *n_all - c0;
+    return left < 0 ? 0 : (left < cap ? left : cap);
+  }
+  __device__ __forceinline__ int64_t token(int r) const {
+    return row_token ? (int64_t)row_token[r] : t0 + r;
+  }
+};
+
 // ----------------------------------------------------------------------------
 // K1: logits tile = lm_head[256 vocab rows] x hidden[256 positions]^T, with
 // per-position (max, sum-exp) partials over the tile's vocab rows, gather of
 // the target logit, and (optionally) the bf16 logits stored to a scratch.
 // ----------------------------------------------------------------------------
 struct FwdParams {
-  const void* hidden;   // [Tc,H] bf16: first row = position t0
+  const void* hidden;   // bf16 [*,H]: dense: first row = position t0; compact: position 0
   const void* W;        // [V,H] bf16
   const int64_t* ids;   // [T] (whole batch)
-  int64_t t0, Tc, T, S, V, H;
+  ChunkRows rows;
+  int64_t Tc;           // row pitch of part / sel (= rows.cap)
+  int64_t S, V, H;
   int shift;
   float2* part;         // [2*VT][Tc]  (max, sumexp)
   float* sel;           // [Tc]        selected logit (pre-filled with NaN)
   uint16_t* stash;      // [Tc,V] bf16 logits or nullptr
-  const uint8_t* need;  // [Tc] rows of the stash that the backward will read
+  const uint8_t* need;  // [Tc] rows of the stash that the backward will read; nullptr: all
   int VT, TT;
 };
 
@@ -63,7 +85,7 @@ struct FwdParams {
 template <bool RAGGED>
 __device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt, int wm,
                                              int64_t vbase, const int64_t (&y)[FWD_NI],
-                                             const int (&col)[FWD_NI]) {
+                                             const int (&col)[FWD_NI], int n) {
   const int lane = threadIdx.x & 63;
   const int half = lane >> 5;
   const int vleft = (int)(p.V - vbase < 128 ? p.V - vbase : 128);  // valid rows of this wave
@@ -91,7 +113,7 @@ __device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const F
         l += (RAGGED && r >= vleft) ? 0.f : e;
       }
     l += __shfl_xor(l, 32, 64);
-    if (lane < 32 && col[ni] < p.Tc)
+    if (lane < 32 && col[ni] < n)
       p.part[(int64_t)(vt * 2 + wm) * p.Tc + col[ni]] = make_float2(m, l);
 
     // Gather: exactly one lane of one wave of the whole grid holds logit[y].
@@ -117,11 +139,13 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   int vt, tt;
   tile_coords(id, p.VT, p.TT, vt, tt);
+  const int n = p.rows.n();
+  if (tt * TILE >= n) return;  // compact mode: token tiles past the last row
 
   TileAcc<FWD_NI> acc;
   acc.zero();
-  gemm_tile_nt(acc, smem, p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE,
-               p.Tc, 0, (int)p.H);
+  gemm_tile_nt(acc, smem, p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0,
+               (int)p.H, p.rows.row_token);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -135,13 +159,13 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
 #pragma unroll
   for (int ni = 0; ni < FWD_NI; ++ni) {
     col[ni] = tt * TILE + acc_col<FWD_NI>(wn, ni, lane);
-    y[ni] = col[ni] < p.Tc ? target_id(p.ids, p.t0 + col[ni], p.S, p.shift) : (int64_t)-1;
+    y[ni] = col[ni] < n ? target_id(p.ids, p.rows.token(col[ni]), p.S, p.shift) : (int64_t)-1;
   }
 
   if (STASH) {
 #pragma unroll
     for (int ni = 0; ni < FWD_NI; ++ni) {
-      const bool want = col[ni] < p.Tc && p.need[col[ni]] != 0;
+      const bool want = col[ni] < n && (p.need == nullptr || p.need[col[ni]] != 0);
       if (!__any(want)) continue;
       if (want) {
         uint16_t* row = p.stash + (int64_t)col[ni] * p.V;
@@ -164,24 +188,26 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
   // The accumulators are only read from here on (writing to them would make the
   // compiler shuttle all 256 between the accumulation and the vector registers).
   if ((int64_t)vt * TILE + TILE > p.V)
-    lse_epilogue<true>(acc, p, vt, wm, vbase, y, col);
+    lse_epilogue<true>(acc, p, vt, wm, vbase, y, col, n);
   else
-    lse_epilogue<false>(acc, p, vt, wm, vbase, y, col);
+    lse_epilogue<false>(acc, p, vt, wm, vbase, y, col, n);
 }
 
 // K2: merge the per-tile (max, sumexp) partials of each position.  A block
 // handles 16 positions; 16 threads per position each merge a strided share of
 // the partials online, then the 16 shares are merged through LDS.
+// logprob is indexed by position (whole batch), lse by chunk row.
 __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restrict__ part,
-                                                           int nparts, int64_t Tc,
+                                                           int nparts, int64_t Tc, ChunkRows rows,
                                                            const float* __restrict__ sel,
                                                            float* __restrict__ logprob,
                                                            float* __restrict__ lse) {
   __shared__ float2 red[16][17];
   const int tl = threadIdx.x & 15, sl = threadIdx.x >> 4;
   const int64_t t = (int64_t)blockIdx.x * 16 + tl;
+  const int n = rows.n();
   float m = -INFINITY, l = 0.f;
-  if (t < Tc) {
+  if (t < n) {
     for (int i = sl; i < nparts; i += 16) {
       const float2 v = part[(int64_t)i * Tc + t];
       const float mn = fmaxf(m, v.x);
@@ -192,7 +218,7 @@ __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restr
   }
   red[sl][tl] = make_float2(m, l);
   __syncthreads();
-  if (sl == 0 && t < Tc) {
+  if (sl == 0 && t < n) {
     float M = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) M = fmaxf(M, red[i][tl].x);
@@ -204,7 +230,7 @@ __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restr
     }
     const float z = M + logf(L);
     lse[t] = z;
-    logprob[t] = sel[t] - z;
+    if (logprob) logprob[rows.token((int)t)] = sel[t] - z;
   }
 }
 
@@ -229,6 +255,49 @@ __global__ __launch_bounds__(256) void need_from_grad_kernel(const float* __rest
                                                              uint8_t* __restrict__ need) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) need[i] = g[i] != 0.f;
+}
+
+// Positions of the whole batch that can have a non-zero loss coefficient (same
+// test as need_from_inputs_kernel), ascending, and their number.  One block.
+__global__ __launch_bounds__(1024) void compact_eval_kernel(const uint8_t* __restrict__ mask,
+                                                            const float* __restrict__ weights,
+                                                            const float* __restrict__ adv,
+                                                            const float* __restrict__ ref_lp, int64_t T,
+                                                            int64_t S, int shift,
+                                                            int* __restrict__ eval_idx,
+                                                            int* __restrict__ n_eval) {
+  __shared__ int wave_tot[16];
+  const int64_t per = (T + 1023) / 1024;
+  const int64_t r0 = threadIdx.x * per;
+  auto wanted = [&](int64_t t) {
+    int64_t src;
+    return shifted_index(t, S, shift, src) && mask[src] != 0 && weights[src] != 0.f &&
+           (adv[src] != 0.f || ref_lp != nullptr);
+  };
+  int cnt = 0;
+  for (int64_t i = 0; i < per; ++i)
+    if (r0 + i < T && wanted(r0 + i)) ++cnt;
+  int incl = cnt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int v = __shfl_up(incl, o, 64);
+    if ((threadIdx.x & 63) >= o) incl += v;
+  }
+  if ((threadIdx.x & 63) == 63) wave_tot[threadIdx.x >> 6] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int w = 0; w < 16; ++w) {
+      int v = wave_tot[w];
+      wave_tot[w] = run;
+      run += v;
+    }
+    *n_eval = run;
+  }
+  __syncthreads();
+  int at = wave_tot[threadIdx.x >> 6] + incl - cnt;
+  for (int64_t i = 0; i < per; ++i)
+    if (r0 + i < T && wanted(r0 + i)) eval_idx[at++] = (int)(r0 + i);
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
@@ -262,32 +331,33 @@ __global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restr
 }
 
 struct LossParams {
-  const float* new_lp;   // [n] position frame, first element = position t0
+  const float* new_lp;   // [T] by position (whole batch)
   const float* old_lp;   // [T] whole batch (frame given by shift)
   const float* adv;      // [T]
   const uint8_t* mask;   // [T]
   const float* weights;  // [T]
-  const float* ref_lp;   // [n] position frame (same origin as new_lp) or nullptr
+  const float* ref_lp;   // [T] by position, or nullptr
   const int* count;      // mask count of the whole batch
-  int64_t t0, n, T, S;
+  ChunkRows rows;
+  int64_t S;
   int shift;
   float clip_lo, clip_hi, beta;
-  float* pl_tok;         // [n] weighted policy-loss term
-  float* kl_tok;         // [n] weighted KL term
-  float* coef;           // [n] d loss / d new_lp, or nullptr
+  float* pl_tok;         // [T] by position: weighted policy-loss term
+  float* kl_tok;         // [T] by position: weighted KL term
+  float* coef;           // [rows.cap] by chunk row: d loss / d new_lp, or nullptr
 };
 
 __global__ __launch_bounds__(256) void grpo_loss_tok_kernel(LossParams p) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= p.n) return;
-  const int64_t t = p.t0 + i;
+  if (i >= p.rows.n()) return;
+  const int64_t t = p.rows.token((int)i);
   int64_t src;
   const bool in = shifted_index(t, p.S, p.shift, src);
   float oldv = in ? p.old_lp[src] : 0.f;
   const float adv = in ? p.adv[src] : 0.f;
   const float w = in ? p.weights[src] : 0.f;
   const float m = (in && p.mask[src] != 0) ? 1.f : 0.f;
-  const float nw = p.new_lp[i];
+  const float nw = p.new_lp[t];
   if (isnan(oldv)) oldv = nw;  // missing old logprob: sampled under the current policy
   const float ratio = expf(nw - oldv);
   const float a = ratio * adv;
@@ -300,15 +370,15 @@ __global__ __launch_bounds__(256) void grpo_loss_tok_kernel(LossParams p) {
   float g = (inside || a < b) ? -a : 0.f;
   float kl = 0.f;
   if (p.ref_lp != nullptr) {
-    const float d = p.ref_lp[i] - nw;
+    const float d = p.ref_lp[t] - nw;
     const float e = expf(d);
     kl = e - d - 1.f;
     g += p.beta * (1.f - e);
   }
   const float denom = (float)(*p.count) + 1e-6f;
   const float wm = w * m;
-  p.pl_tok[i] = pl * wm;
-  p.kl_tok[i] = kl * wm;
+  p.pl_tok[t] = pl * wm;
+  p.kl_tok[t] = kl * wm;
   if (p.coef) p.coef[i] = (wm != 0.f) ? g * wm / denom : 0.f;
 }
 
@@ -355,14 +425,16 @@ __global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __r
 //   sched[0] = n_active, [1] = token tiles, [2] = K splits, [3] = work-groups
 // Rows whose coefficient is zero (non-assistant positions, zero advantage) have
 // an exactly zero d_hidden row and are skipped by K3b and K4.
-__global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restrict__ coef, int Tc,
-                                                            int HT, int ksteps, int part_rows,
+__global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restrict__ coef,
+                                                            ChunkRows rows, int HT, int ksteps,
+                                                            int part_rows,
                                                             int num_cus, int* __restrict__ active_idx,
                                                             int* __restrict__ pos,
                                                             int* __restrict__ sched) {
   __shared__ int wave_tot[16];
   __shared__ int total;
-  const int per = (Tc + 1023) / 1024;
+  const int Tc = rows.n();
+  const int per = (rows.cap + 1023) / 1024;
   const int r0 = threadIdx.x * per;
   int cnt = 0;
   for (int i = 0; i < per; ++i) {
@@ -430,7 +502,7 @@ __global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict_
                                                            const float* __restrict__ lse,
                                                            const float* __restrict__ coef,
                                                            const int64_t* __restrict__ ids,
-                                                           int64_t t0, int64_t S, int shift,
+                                                           ChunkRows rows, int64_t S, int shift,
                                                            const int* __restrict__ active_idx,
                                                            const int* __restrict__ sched) {
   if ((int)blockIdx.x >= sched[0]) return;
@@ -438,7 +510,7 @@ __global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict_
   uint4* row = (uint4*)(stash + r * V);
   const int nvec = (int)(V >> 3);
   const float c = coef[r];
-  const int64_t y = target_id(ids, t0 + r, S, shift);
+  const int64_t y = target_id(ids, rows.token((int)r), S, shift);
   const float nl = -lse[r] * LOG2E;
   for (int i = threadIdx.x; i < nvec; i += 256) {
     uint4 x = row[i];
@@ -515,15 +587,17 @@ __global__ __launch_bounds__(nthreads<BWD_NI>()) void dhidden_gemm_kernel(BwdPar
   }
 }
 
-// K5: d_hidden row r = bf16(sum over splits of partial[compact row of r]) or 0
-// for inactive rows; 4 elements per thread.
+// K5: d_hidden row of chunk row r = bf16(sum over splits of partial[active slot
+// of r]) or 0 for inactive rows; 4 elements per thread.  `out` is the whole
+// batch's d_hidden, indexed by position.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
                                                             const int* __restrict__ pos,
-                                                            const int* __restrict__ sched, int64_t Tc,
-                                                            int64_t H, uint16_t* __restrict__ out) {
+                                                            const int* __restrict__ sched,
+                                                            ChunkRows rows, int64_t H,
+                                                            uint16_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t h4 = H / 4;
-  if (i >= Tc * h4) return;
+  if (i >= (int64_t)rows.n() * h4) return;
   const int64_t r = i / h4, c = i - r * h4;
   const int pr = pos[r];
   floatx4 s = {0.f, 0.f, 0.f, 0.f};
@@ -536,7 +610,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   bf16x4 o;
 #pragma unroll
   for (int e = 0; e < 4; ++e) o[e] = (__bf16)s[e];
-  ((bf16x4*)out)[i] = o;
+  ((bf16x4*)out)[rows.token((int)r) * h4 + c] = o;
 }
 
 // ----------------------------------------------------------------------------
@@ -662,19 +736,29 @@ static int32_t check_common(const void* hidden, const void* lm_head, int64_t T, 
   return ARTK_OK;
 }
 
-// Launch K1 (+ NaN pre-fill of sel) and K2 for positions [t0, t0+Tc).
+static ChunkRows dense_rows(int64_t t0, int64_t n) {
+  ChunkRows r;
+  r.row_token = nullptr;
+  r.n_all = nullptr;
+  r.t0 = t0;
+  r.c0 = 0;
+  r.cap = (int)n;
+  return r;
+}
+
+// Launch K1 (+ NaN pre-fill of sel) and K2 for the rows of one chunk.  `logprob`
+// (may be null) is the whole batch's array; `lse_chunk` is indexed by chunk row.
 static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const int64_t* ids,
-                                int shift, int64_t t0, int64_t Tc, int64_t T, int64_t S, int64_t V,
-                                int64_t H, float2* part, float* sel, uint16_t* stash,
-                                const uint8_t* need, float* logprob_chunk, float* lse_chunk,
-                                hipStream_t st) {
+                                int shift, const ChunkRows& rows, int64_t S, int64_t V, int64_t H,
+                                float2* part, float* sel, uint16_t* stash, const uint8_t* need,
+                                float* logprob, float* lse_chunk, hipStream_t st) {
+  const int64_t Tc = rows.cap;
   FwdParams p;
-  p.hidden = (const char*)hidden + t0 * H * 2;
+  p.hidden = rows.row_token ? hidden : (const void*)((const char*)hidden + rows.t0 * H * 2);
   p.W = lm_head;
   p.ids = ids;
-  p.t0 = t0;
+  p.rows = rows;
   p.Tc = Tc;
-  p.T = T;
   p.S = S;
   p.V = V;
   p.H = H;
@@ -695,8 +779,8 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
     lmhead_fwd_kernel<false><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
   prof_end(PROF_LMHEAD_FWD, st);
   ARTK_CHECK_LAUNCH();
-  lse_finalize_kernel<<<(unsigned)((Tc + 15) / 16), 256, 0, st>>>(part, 2 * p.VT, Tc, sel,
-                                                                    logprob_chunk, lse_chunk);
+  lse_finalize_kernel<<<(unsigned)((Tc + 15) / 16), 256, 0, st>>>(part, 2 * p.VT, Tc, rows, sel, logprob,
+                                                                    lse_chunk);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -718,18 +802,20 @@ struct BwdScratch {
 };
 
 // Launch K3a, K3b, K4, K5 for one chunk whose bf16 logits are in `stash`.
+// `d_hidden` is the whole batch's gradient, indexed by position.
 static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const int64_t* ids,
-                                int shift, int64_t t0, int64_t Tc, int64_t S, int64_t V, int64_t H,
+                                int shift, const ChunkRows& rows, int64_t S, int64_t V, int64_t H,
                                 const float* lse_chunk, const float* coef_chunk, const BwdScratch& sc,
-                                uint16_t* d_hidden_chunk, hipStream_t st) {
+                                uint16_t* d_hidden, hipStream_t st) {
+  const int64_t Tc = rows.cap;
   const int HT = (int)((H + TILE - 1) / TILE);
   const int TT = (int)((Tc + TILE - 1) / TILE);
-  compact_rows_kernel<<<1, 1024, 0, st>>>(coef_chunk, (int)Tc, HT, (int)(V / BK), (int)sc.part_rows,
+  compact_rows_kernel<<<1, 1024, 0, st>>>(coef_chunk, rows, HT, (int)(V / BK), (int)sc.part_rows,
                                           num_cus(), sc.active_idx, sc.pos, sc.sched);
   ARTK_CHECK_LAUNCH();
   prof_begin(PROF_SOFTMAX_GRAD, st);
-  softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, t0, S,
-                                                    shift, sc.active_idx, sc.sched);
+  softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, rows, S, shift,
+                                                    sc.active_idx, sc.sched);
   prof_end(PROF_SOFTMAX_GRAD, st);
   ARTK_CHECK_LAUNCH();
   BwdParams b;
@@ -749,8 +835,8 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   prof_end(PROF_DHIDDEN_GEMM, st);
   ARTK_CHECK_LAUNCH();
   const int64_t n4 = Tc * H / 4;
-  splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(sc.partial, sc.pos, sc.sched, Tc,
-                                                                     H, d_hidden_chunk);
+  splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(sc.partial, sc.pos, sc.sched, rows,
+                                                                     H, d_hidden);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -785,8 +871,8 @@ int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t*
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
-  return launch_fwd_chunk(hidden, lm_head, ids, shift, 0, T, T, S, V, H, part, sel, nullptr, nullptr,
-                          logprob, lse, (hipStream_t)stream);
+  return launch_fwd_chunk(hidden, lm_head, ids, shift, dense_rows(0, T), S, V, H, part, sel, nullptr,
+                          nullptr, logprob, lse, (hipStream_t)stream);
 }
 
 // Scratch of one chunk of Tc positions carved out of the caller's workspace.
@@ -796,9 +882,12 @@ struct ChunkScratch {
   float* sel;       // [Tc]
   uint8_t* need;    // [Tc]
   BwdScratch bwd;
-  float *lse, *coef, *pl, *kl;  // [T] each (fused op only)
+  float *lse, *coef;            // [Tc] each, by chunk row (fused op only)
+  float *pl, *kl;               // [T] each, by position (fused op only)
   int* count;
-  float *lp_tmp, *lse_tmp;      // [Tc] each (standalone backward only)
+  int* eval_idx;                // [T] positions the forward is evaluated for (fused op, skip mode)
+  int* n_eval;
+  float* lse_tmp;               // [Tc] (standalone backward only)
 };
 
 static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bool fused,
@@ -814,13 +903,14 @@ static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bo
   c.bwd.pos = ws.take<int>((size_t)Tc);
   c.bwd.sched = ws.take<int>(64);
   if (fused) {
-    c.lse = ws.take<float>((size_t)T);
-    c.coef = ws.take<float>((size_t)T);
+    c.lse = ws.take<float>((size_t)Tc);
+    c.coef = ws.take<float>((size_t)Tc);
     c.pl = ws.take<float>((size_t)T);
     c.kl = ws.take<float>((size_t)T);
     c.count = ws.take<int>(64);
+    c.eval_idx = ws.take<int>((size_t)T);
+    c.n_eval = ws.take<int>(64);
   } else {
-    c.lp_tmp = ws.take<float>((size_t)Tc);
     c.lse_tmp = ws.take<float>((size_t)Tc);
   }
 }
@@ -872,11 +962,12 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
     // The scratch row pitch is V, so a shorter last chunk simply uses fewer rows.
     need_from_grad_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(grad_logprob + t0, n, c.need);
     ARTK_CHECK_LAUNCH();
-    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, t0, n, T, S, V, H, c.part, c.sel, c.stash,
-                          c.need, c.lp_tmp, c.lse_tmp, st);
+    const ChunkRows rows = dense_rows(t0, n);
+    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, rows, S, V, H, c.part, c.sel, c.stash, c.need,
+                          nullptr, c.lse_tmp, st);
     if (rc) return rc;
-    rc = launch_bwd_chunk(c.stash, lm_head_t, ids, shift, t0, n, S, V, H, lse + t0,
-                          grad_logprob + t0, c.bwd, (uint16_t*)d_hidden + t0 * H, st);
+    rc = launch_bwd_chunk(c.stash, lm_head_t, ids, shift, rows, S, V, H, lse + t0, grad_logprob + t0,
+                          c.bwd, (uint16_t*)d_hidden, st);
     if (rc) return rc;
   }
   return ARTK_OK;
@@ -897,7 +988,7 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
                        artk_stream_t stream) {
   ARTK_CHECK_ARG(new_logprob && old_logprob && advantages && mask && weights && scalars,
                  "null pointer argument");
-  ARTK_CHECK_ARG(T > 0 && S > 0 && T % S == 0, "T must be a positive multiple of S");
+  ARTK_CHECK_ARG(T > 0 && S > 0 && T % S == 0 && T < (1ll << 31), "T must be a positive multiple of S below 2^31");
   ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
   ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
   Workspace ws(workspace, workspace_bytes);
@@ -919,9 +1010,7 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
   p.weights = weights;
   p.ref_lp = (beta > 0.f) ? ref_logprob : nullptr;
   p.count = count;
-  p.t0 = 0;
-  p.n = T;
-  p.T = T;
+  p.rows = dense_rows(0, T);
   p.S = S;
   p.shift = shift;
   p.clip_lo = clip_lo;
@@ -948,8 +1037,8 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
                         const int64_t* tokens, const float* old_logprob, const float* advantages,
                         const uint8_t* mask, const float* weights, const float* ref_logprob,
                         int64_t T, int64_t S, int64_t V, int64_t H, float clip_lo, float clip_hi,
-                        float beta, int64_t chunk_tokens, float* scalars, float* logprob,
-                        void* d_hidden, void* workspace, size_t workspace_bytes,
+                        float beta, int64_t chunk_tokens, int32_t flags, float* scalars,
+                        float* logprob, void* d_hidden, void* workspace, size_t workspace_bytes,
                         artk_stream_t stream) {
   int32_t rc = check_common(hidden, lm_head, T, S, V, H, true);
   if (rc) return rc;
@@ -958,6 +1047,13 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
                  "null pointer argument");
   ARTK_CHECK_ARG(aligned16(lm_head_t) && aligned16(d_hidden), "pointers must be 16-byte aligned");
   ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
+  ARTK_CHECK_ARG((flags & ~ARTK_FUSED_SKIP_INACTIVE) == 0, "unknown flag bits 0x%x", (unsigned)flags);
+  const bool skip = (flags & ARTK_FUSED_SKIP_INACTIVE) != 0;
+  if (skip && T * H * 2 >= (1ll << 31)) {
+    // gathered rows of `hidden` are addressed with 31-bit byte offsets
+    set_error("ARTK_FUSED_SKIP_INACTIVE needs T*H*2 < 2^31 bytes of hidden states");
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
   const int64_t Tc = clamp_chunk(T, V, chunk_tokens);
   Workspace ws(workspace, workspace_bytes);
   ChunkScratch c;
@@ -970,37 +1066,63 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
   const float* ref = (beta > 0.f) ? ref_logprob : nullptr;
   mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, 1, c.count);
   ARTK_CHECK_LAUNCH();
-  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
-    const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
-    need_from_inputs_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(mask, weights, advantages,
-                                                                         ref, t0, n, S, 1, c.need);
+  if (skip) {
+    // Positions that are not evaluated keep: logprob NaN, zero loss terms, zero d_hidden.
+    compact_eval_kernel<<<1, 1024, 0, st>>>(mask, weights, advantages, ref, T, S, 1, c.eval_idx,
+                                            c.n_eval);
     ARTK_CHECK_LAUNCH();
-    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, t0, n, T, S, V, H, c.part, c.sel, c.stash,
-                          c.need, logprob + t0, c.lse + t0, st);
+    const unsigned gT = (unsigned)((T + 255) / 256);
+    fill_f32_kernel<<<gT, 256, 0, st>>>(logprob, T, NAN);
+    ARTK_CHECK_LAUNCH();
+    fill_f32_kernel<<<gT, 256, 0, st>>>(c.pl, T, 0.f);
+    ARTK_CHECK_LAUNCH();
+    fill_f32_kernel<<<gT, 256, 0, st>>>(c.kl, T, 0.f);
+    ARTK_CHECK_LAUNCH();
+    const int64_t nd = T * H / 2;  // bf16 pairs
+    fill_f32_kernel<<<(unsigned)((nd + 255) / 256), 256, 0, st>>>((float*)d_hidden, nd, 0.f);
+    ARTK_CHECK_LAUNCH();
+  }
+  // In skip mode the number of evaluated rows is known only on the device: every
+  // chunk the worst case needs is launched and the ones past the end do nothing.
+  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
+    ChunkRows rows;
+    if (skip) {
+      rows.row_token = c.eval_idx + t0;
+      rows.n_all = c.n_eval;
+      rows.t0 = 0;
+      rows.c0 = (int)t0;
+      rows.cap = (int)Tc;
+    } else {
+      const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
+      rows = dense_rows(t0, n);
+      need_from_inputs_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(mask, weights, advantages,
+                                                                           ref, t0, n, S, 1, c.need);
+      ARTK_CHECK_LAUNCH();
+    }
+    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, rows, S, V, H, c.part, c.sel, c.stash,
+                          skip ? nullptr : c.need, logprob, c.lse, st);
     if (rc) return rc;
     LossParams p;
-    p.new_lp = logprob + t0;
+    p.new_lp = logprob;
     p.old_lp = old_logprob;
     p.adv = advantages;
     p.mask = mask;
     p.weights = weights;
-    p.ref_lp = ref ? ref + t0 : nullptr;
+    p.ref_lp = ref;
     p.count = c.count;
-    p.t0 = t0;
-    p.n = n;
-    p.T = T;
+    p.rows = rows;
     p.S = S;
     p.shift = 1;
     p.clip_lo = clip_lo;
     p.clip_hi = clip_hi;
     p.beta = beta;
-    p.pl_tok = c.pl + t0;
-    p.kl_tok = c.kl + t0;
-    p.coef = c.coef + t0;
-    grpo_loss_tok_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(p);
+    p.pl_tok = c.pl;
+    p.kl_tok = c.kl;
+    p.coef = c.coef;
+    grpo_loss_tok_kernel<<<(unsigned)((rows.cap + 255) / 256), 256, 0, st>>>(p);
     ARTK_CHECK_LAUNCH();
-    rc = launch_bwd_chunk(c.stash, lm_head_t, tokens, 1, t0, n, S, V, H, c.lse + t0, c.coef + t0,
-                          c.bwd, (uint16_t*)d_hidden + t0 * H, st);
+    rc = launch_bwd_chunk(c.stash, lm_head_t, tokens, 1, rows, S, V, H, c.lse, c.coef, c.bwd,
+                          (uint16_t*)d_hidden, st);
     if (rc) return rc;
   }
   grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(c.pl, c.kl, T, c.count, ref ? beta : 0.f, scalars);

@@ -14,6 +14,7 @@ import torch
 from . import _lib
 
 DEFAULT_CHUNK_TOKENS = 0  # 0: the library picks (about 6000 positions, split evenly)
+FUSED_SKIP_INACTIVE = 1   # ARTK_FUSED_SKIP_INACTIVE
 
 
 def _stream(device) -> int:
@@ -191,11 +192,13 @@ def grpo_loss(new_logprob, old_logprob, advantages, mask, weights, ref_logprob, 
 def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask, weights,
                ref_logprob, row_len: int, clip_lo: float, clip_hi: float, beta: float,
                chunk_tokens: int = DEFAULT_CHUNK_TOKENS, workspace: Optional[torch.Tensor] = None,
-               out: Optional[tuple] = None):
+               out: Optional[tuple] = None, skip_inactive: bool = False):
     """One call for loss and d_hidden of a packed batch given its hidden states.
 
     All per-token inputs are the un-shifted PackedTensors rows flattened to [T].
-    Returns (scalars f32 [4], logprob f32 [T], d_hidden bf16 [T,H])."""
+    Returns (scalars f32 [4], logprob f32 [T], d_hidden bf16 [T,H]).  With
+    skip_inactive the lm_head projection runs only for positions that can
+    contribute to the loss; logprob is NaN elsewhere."""
     T, H = hidden.shape
     V = lm_head.shape[0]
     _need(hidden, "hidden", torch.bfloat16)
@@ -222,7 +225,8 @@ def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask
         lib.artk_grpo_fused(hidden.data_ptr(), lm_head.data_ptr(), lm_head_t.data_ptr(),
                             tokens.data_ptr(), old_logprob.data_ptr(), advantages.data_ptr(),
                             mask.data_ptr(), weights.data_ptr(), _ptr(ref_logprob), T, row_len, V,
-                            H, clip_lo, clip_hi, beta, chunk_tokens, scalars.data_ptr(),
+                            H, clip_lo, clip_hi, beta, chunk_tokens,
+                            FUSED_SKIP_INACTIVE if skip_inactive else 0, scalars.data_ptr(),
                             logprob.data_ptr(), d_hidden.data_ptr(), ws.data_ptr(), ws.numel(),
                             _stream(dev))
     )

@@ -161,13 +161,14 @@ class _FusedGRPOLossFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, lm_head, tokens, old, adv, mask, weights, ref, clip_lo, clip_hi, beta,
-                chunk_tokens):
+                chunk_tokens, skip_inactive):
         B, S, H = hidden.shape
         T = B * S
         flat = lambda t: None if t is None else t.reshape(T).contiguous()
         scalars, logprob, d_hidden = ops.grpo_fused(
             hidden.reshape(T, H), lm_head, ops.transposed_weight(lm_head), flat(tokens), flat(old),
-            flat(adv), flat(mask), flat(weights), flat(ref), S, clip_lo, clip_hi, beta, chunk_tokens)
+            flat(adv), flat(mask), flat(weights), flat(ref), S, clip_lo, clip_hi, beta, chunk_tokens,
+            skip_inactive=skip_inactive)
         ctx.save_for_backward(d_hidden)
         ctx.shape = (B, S, H)
         logprob = logprob.view(B, S)
@@ -178,24 +179,29 @@ class _FusedGRPOLossFn(torch.autograd.Function):
     def backward(ctx, g_loss, _g_scalars, _g_logprob):
         (d_hidden,) = ctx.saved_tensors
         g = (d_hidden * g_loss).to(d_hidden.dtype).view(ctx.shape)
-        return (g,) + (None,) * 11
+        return (g,) + (None,) * 12
 
 
 def fused_grpo_loss(hidden_states, lm_head, tokens, logprobs, advantages, assistant_mask, weights,
                     epsilon=0.2, epsilon_high=None, ref_logprobs=None, beta=0.0,
-                    chunk_tokens: int = ops.DEFAULT_CHUNK_TOKENS):
+                    chunk_tokens: int = ops.DEFAULT_CHUNK_TOKENS, skip_inactive: bool = False):
     """Loss of one packed batch from the model's hidden states, in one library call.
 
     Takes the *un-shifted* PackedTensors rows ([B, S]); equivalent to
     ``shift_tensor`` x5 + ``_calculate_logprobs`` + ``grpo_loss`` of the reference
-    (src/art/local/train.py:76-151).  Returns (loss, metrics, new_logprobs)."""
+    (src/art/local/train.py:76-151).  Returns (loss, metrics, new_logprobs).
+
+    ``skip_inactive``: project only the positions whose loss term can be
+    non-zero (the reference projects all of them and multiplies by the mask,
+    train.py:145-151); loss, metrics and gradient are unchanged, new_logprobs is
+    NaN at the skipped positions."""
     clip_lo, clip_hi = ops.clip_bounds(epsilon, epsilon_high)
     ref = ref_logprobs if beta > 0.0 else None
     hidden = hidden_states.to(torch.bfloat16).contiguous()
     loss, scalars, logprob = _FusedGRPOLossFn.apply(
         hidden, lm_head, tokens, logprobs.to(torch.float32), advantages.to(torch.float32),
         assistant_mask, weights.to(torch.float32), None if ref is None else ref.to(torch.float32),
-        clip_lo, clip_hi, float(beta), chunk_tokens)
+        clip_lo, clip_hi, float(beta), chunk_tokens, bool(skip_inactive))
     return loss, {"policy_loss": scalars[1], "kl_div": scalars[2], "mask_count": scalars[3]}, logprob
 
 
@@ -255,7 +261,7 @@ def get_compute_loss_fn(trainer) -> Callable[..., torch.Tensor]:
         loss, metrics, _ = fused_grpo_loss(
             hidden_states, lm_head.detach().to(torch.bfloat16), inputs["tokens"], inputs["logprobs"],
             inputs["advantages"], inputs["assistant_mask"], inputs["weights"], epsilon, epsilon_high,
-            ref_logprobs, config.beta)
+            ref_logprobs, config.beta, skip_inactive=True)  # new_logprobs are not used here
 
         trainer._metrics["learning_rate"].append(config.learning_rate)
         trainer._metrics["policy_loss"].append(metrics["policy_loss"].item())

@@ -279,9 +279,9 @@ def main():
            torch.empty(T, dtype=torch.float32, device=dev),
            torch.empty((T, H), dtype=torch.bfloat16, device=dev))
 
-    def step():
+    def step(skip_inactive=False):
         ops.grpo_fused(hidden, lm_head, lm_head_t, tokens, old, adv, mask, weights, None, T, 0.8,
-                       1.2, 0.0, chunk, workspace=ws, out=out)
+                       1.2, 0.0, chunk, workspace=ws, out=out, skip_inactive=skip_inactive)
 
     if args.copy_calibration_mib:
         n = args.copy_calibration_mib << 20
@@ -304,6 +304,20 @@ def main():
     bwd_ms, bwd_n = ops.profile_collect(ops.PROF_DHIDDEN_GEMM)
     sm_ms, sm_n = ops.profile_collect(ops.PROF_SOFTMAX_GRAD)
     ops.profile_enable(False)
+    t_active_dense = int(out[0][3].item())
+
+    # Secondary figure (never `value`): the same batch with the projection restricted to the
+    # positions that can contribute to the loss; same loss and gradient, less work.
+    for _ in range(args.warmup):
+        step(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    dt_skip = time.perf_counter() - t0
+    step()  # leave the dense results in `out`
+    torch.cuda.synchronize()
 
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T / (dt / args.steps)
@@ -357,6 +371,10 @@ def main():
             "softmax_grad_kernel": {"launch_ms": sm_ms / max(sm_n, 1)},
         },
     }
+    assert t_active == t_active_dense
+    result["skip_inactive"] = {"value": T / (dt_skip / args.steps), "unit": "tokens/s",
+                               "ms_per_step": dt_skip / args.steps * 1e3,
+                               "note": "flag ARTK_FUSED_SKIP_INACTIVE; batch tokens per second"}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens)
     print(json.dumps(result))

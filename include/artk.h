@@ -107,15 +107,22 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
  *     the shift of train.py:79,112-117 is applied by index arithmetic.
  *   ref_logprob f32 [T] or NULL   (position frame)
  *   scalars f32 [4] out, logprob f32 [T] out, d_hidden bf16 [T,H] out
+ *   flags: 0, or ARTK_FUSED_SKIP_INACTIVE: evaluate the lm_head projection only
+ *     for positions that can contribute to the loss (shifted assistant mask set,
+ *     weight != 0, and advantage != 0 or a KL term).  The reference computes
+ *     logprobs for every position and multiplies the rest by a zero mask
+ *     (train.py:111-151); loss, metrics and d_hidden are the same, but logprob
+ *     of a skipped position is NaN.  Needs T*H*2 < 2^31.
  * Requires H % 64 == 0, V % 64 == 0.
  * ------------------------------------------------------------------------- */
+#define ARTK_FUSED_SKIP_INACTIVE 1
 size_t artk_grpo_fused_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens);
 int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_head_t,
                         const int64_t* tokens, const float* old_logprob, const float* advantages,
                         const uint8_t* mask, const float* weights, const float* ref_logprob,
                         int64_t T, int64_t S, int64_t V, int64_t H, float clip_lo, float clip_hi,
-                        float beta, int64_t chunk_tokens, float* scalars, float* logprob,
-                        void* d_hidden, void* workspace, size_t workspace_bytes,
+                        float beta, int64_t chunk_tokens, int32_t flags, float* scalars,
+                        float* logprob, void* d_hidden, void* workspace, size_t workspace_bytes,
                         artk_stream_t stream);
 
 /* out[c,r] = in[r,c] for a bf16 [R,C] matrix (R, C multiples of 8).  Used once

@@ -22,7 +22,7 @@ def test_header_symbols_are_exported_and_bound(artk_lib):
     for n in names:
         assert hasattr(artk_lib, n), f"{n} declared in artk.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
-    assert artk_lib.artk_abi_version() == 1
+    assert artk_lib.artk_abi_version() == 2
 
 
 def test_argument_errors_have_codes_and_messages(artk_lib):

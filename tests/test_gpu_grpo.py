@@ -182,6 +182,61 @@ def test_fused_all_or_no_rows_active(artk_lib, gpu, density):
         assert metrics["mask_count"].item() == T - 1  # the last position's mask shifts out
 
 
+@pytest.mark.parametrize("T,H,V,n_traj,chunk_tokens,density,beta",
+                         [(512, 256, 8192, 4, 4096, 0.5, 0.0), (1024, 128, 4096, 8, 256, 0.3, 0.0),
+                          (768, 192, 8000, 4, 256, 0.5, 0.05), (512, 128, 4096, 4, 256, 0.0, 0.0),
+                          (512, 128, 4096, 4, 256, 1.0, 0.0)])
+def test_fused_skip_inactive(artk_lib, gpu, T, H, V, n_traj, chunk_tokens, density, beta):
+    """Projecting only the positions that can contribute gives the oracle's loss
+    and gradient, the dense mode's loss bit for bit, and NaN logprobs exactly at
+    the skipped positions."""
+    print(f"fused skip T={T} H={H} V={V} chunk={chunk_tokens} density={density} beta={beta}", flush=True)
+    case = synthetic.make_grpo_case("t", T + H + 1, T, H, V, n_traj, 4, 0.5)
+    if density in (0.0, 1.0):
+        from art_amd.advantage import token_weights
+        case.assistant_mask = torch.full_like(case.assistant_mask, bool(density))
+        case.weights = (token_weights(case.assistant_mask, case.traj_id) if density
+                        else torch.zeros_like(case.weights))
+    oracle_case(case, T // 2)
+    ref_lp = None
+    if beta > 0:
+        g = torch.Generator().manual_seed(11)
+        ref_lp = grpo_oracle.shift_tensor(
+            case.logprobs.nan_to_num(-8.0) + 0.1 * torch.randn(1, T, generator=g), 0.0)
+    ref = grpo_oracle.loss_and_grad(case.hidden, case.lm_head, case.tokens, case.logprobs,
+                                    case.advantages, case.assistant_mask, case.weights,
+                                    chunk_size=T // 2, ref_logprobs=ref_lp, beta=beta)
+    res = {}
+    for skip in (False, True):
+        hidden = case.hidden.to(gpu).requires_grad_(True)
+        loss, metrics, logprob = fused_grpo_loss(
+            hidden, case.lm_head.to(gpu), case.tokens.to(gpu), case.logprobs.to(gpu),
+            case.advantages.to(gpu), case.assistant_mask.to(gpu), case.weights.to(gpu),
+            ref_logprobs=None if ref_lp is None else ref_lp.to(gpu), beta=beta,
+            chunk_tokens=chunk_tokens, skip_inactive=skip)
+        loss.backward()
+        res[skip] = (loss.detach().cpu(), metrics, logprob.cpu(), hidden.grad.float().cpu())
+    loss, metrics, logprob, grad = res[True]
+    assert torch.equal(loss, res[False][0])
+    assert torch.equal(metrics["policy_loss"].cpu(), res[False][1]["policy_loss"].cpu())
+    assert torch.equal(metrics["kl_div"].cpu(), res[False][1]["kl_div"].cpu())
+    assert metrics["mask_count"].item() == res[False][1]["mask_count"].item()
+    # which positions are evaluated
+    sh = lambda t, fill: grpo_oracle.shift_tensor(t, fill)
+    want = sh(case.assistant_mask, False) & (sh(case.weights, 0.0) != 0)
+    if beta == 0:
+        want &= sh(case.advantages, 0.0) != 0
+    assert torch.equal(~torch.isnan(logprob), want)
+    assert torch.equal(logprob[want], res[False][2][want])
+    if density == 0.0:
+        assert loss.item() == 0.0 and grad.abs().max().item() == 0.0
+        return
+    assert abs(loss.item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item())
+    assert rel_l2(grad, ref["d_hidden"]) <= GRAD_TOL
+    assert rel_l2(grad, res[False][3]) <= 2e-3  # bf16 rounding of differently ordered fp32 sums
+    assert grad[0][~want[0]].abs().max().item() == 0.0
+
+
 def test_config1_full_size(artk_lib, gpu):
     """BASELINE config 1 (Qwen2.5-0.5B shape) at full size against the oracle."""
     print("config1 full size", flush=True)
@@ -274,3 +329,10 @@ def test_full_size_windows_and_properties(artk_lib, gpu, name):
         grpo_oracle.shift_tensor(case.assistant_mask, False).float(),
         grpo_oracle.shift_tensor(case.weights, 0.0))
     assert abs(s[0].item() - loss_ref.item()) <= LOSS_TOL * abs(loss_ref.item())
+    # skipping the positions that cannot contribute: same loss bit for bit, same gradient
+    s4, lp4, dh4 = ops.grpo_fused(*args, 4096, skip_inactive=True)
+    assert torch.equal(s4, s)
+    assert torch.equal(torch.isnan(lp4), dead.to(gpu))
+    assert torch.equal(lp4[(~dead).to(gpu)], lp[(~dead).to(gpu)])
+    assert rel_l2(dh4.float(), dh.float()) <= 2e-3
+    assert dh4[dead.to(gpu)].abs().max().item() == 0.0
