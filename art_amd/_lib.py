@@ -56,6 +56,11 @@ SIGNATURES = {
     "artk_moe_lora_grouped_bwd": (
         _i32, [_p, _p, _p, _p, _p, _p, _p, _f32, _p, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _p, _p,
                _p, _sz, _p]),
+    "artk_attn_plan_bytes": (_sz, [_i64]),
+    "artk_attn_plan": (_i32, [_p, _p, _i64, _p, _sz, _p]),
+    "artk_attn_fwd_workspace_bytes": (_sz, [_i64, _i32, _i32]),
+    "artk_attn_fwd": (
+        _i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32] + [_i64] * 8 + [_f32, _p, _p, _p, _sz, _p]),
     "artk_transpose_bf16_batched": (_i32, [_p, _p, _i64, _i64, _i64, _p]),
     "artk_profile_enable": (_i32, [_i32]),
     "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),

@@ -381,9 +381,62 @@ def moe_lora_grouped_bwd(g, x, gather, W_t, A, B, xa, scale: float, routing: Rou
 
 
 # -----------------------------------------------------------------------------
+# Packed-row attention
+# -----------------------------------------------------------------------------
+class AttnPlan:
+    """Device-side description of one packed row's visibility (see artk_attn_plan)."""
+
+    __slots__ = ("buf", "S")
+
+
+def attn_plan(group_ids: torch.Tensor, parent_ids: torch.Tensor) -> AttnPlan:
+    """Plan for one packed row: ids are the int64 [S] PackedTensors rows."""
+    S = group_ids.numel()
+    _need(group_ids, "group_ids", torch.int64, (S,))
+    _need(parent_ids, "parent_ids", torch.int64, (S,))
+    lib = _lib.load()
+    dev = group_ids.device
+    plan = AttnPlan()
+    plan.S = S
+    plan.buf = torch.empty(lib.artk_attn_plan_bytes(S), dtype=torch.uint8, device=dev)
+    _lib.check(lib.artk_attn_plan(group_ids.data_ptr(), parent_ids.data_ptr(), S, plan.buf.data_ptr(),
+                                  plan.buf.numel(), _stream(dev)))
+    return plan
+
+
+def _shd(t: torch.Tensor, name: str):
+    """(stride_s, stride_h) of a bf16 [S, H, D] view whose last dimension is contiguous."""
+    if t.dtype != torch.bfloat16 or t.dim() != 3 or t.stride(2) != 1 or not t.is_cuda:
+        raise ValueError(f"{name}: expected a bf16 device tensor [S, H, D] with contiguous D")
+    return t.stride(0), t.stride(1)
+
+
+def attn_fwd(q, k, v, plan: AttnPlan, scale: Optional[float] = None):
+    """(out bf16 [S, Hq, D], lse f32 [Hq, S]) for q [S, Hq, D], k/v [S, Hkv, D] (any strides over S, H)."""
+    S, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != (S, Hkv, D) or v.shape != (S, Hkv, D) or plan.S != S:
+        raise ValueError("attn_fwd: inconsistent shapes")
+    qs, ks, vs = _shd(q, "q"), _shd(k, "k"), _shd(v, "v")
+    lib = _lib.load()
+    dev = q.device
+    out = torch.empty((S, Hq, D), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((Hq, S), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_attn_fwd_workspace_bytes(S, Hkv, D), dev)
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    _lib.check(
+        lib.artk_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), plan.buf.data_ptr(), S, Hq, Hkv, D,
+                          qs[0], qs[1], ks[0], ks[1], vs[0], vs[1], out.stride(0), out.stride(1), scale,
+                          out.data_ptr(), lse.data_ptr(), ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return out, lse
+
+
+# -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------
-PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM = range(5)
+(PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM, PROF_ATTN_FWD,
+ PROF_ATTN_BWD_KV, PROF_ATTN_BWD_Q) = range(8)
 
 
 def profile_enable(on: bool) -> None:

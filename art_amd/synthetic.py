@@ -116,3 +116,28 @@ def config4() -> GRPOCase:
     20-70 % mask per trajectory, Bernoulli rewards."""
     return make_grpo_case("C4-qwen2.5-14b", 1004, 32768, 5120, 152064, 16, 4, (0.2, 0.5),
                           rewards="bernoulli")
+
+
+def packed_row_ids(seed: int, S: int, n_prompts: int, prompt_len: int, n_completions: int,
+                   completion_len: int):
+    """group_ids / parent_ids (int64 [S]) of one packed row the way the packer lays
+    it out (reference: src/art/local/pack.py:84-93, 139-140): each prompt's tokens
+    carry group = parent = prompt id; each of its completions gets a fresh random
+    64-bit group id and parent = prompt id; the tail of the row is padding (-1, -1)."""
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(-(2 ** 62), 2 ** 62, (n_prompts * (1 + n_completions),), generator=g)
+    group, parent = [], []
+    k = 0
+    for _ in range(n_prompts):
+        pid = int(ids[k]); k += 1
+        group += [pid] * prompt_len
+        parent += [pid] * prompt_len
+        for _ in range(n_completions):
+            cid = int(ids[k]); k += 1
+            group += [cid] * completion_len
+            parent += [pid] * completion_len
+    assert len(group) <= S, "row too short for the requested layout"
+    pad = S - len(group)
+    group += [-1] * pad
+    parent += [-1] * pad
+    return torch.tensor(group, dtype=torch.int64), torch.tensor(parent, dtype=torch.int64)

@@ -213,6 +213,37 @@ int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_
                                     artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * Packed-row attention without the dense bias.
+ * Replaces: calculate_attn_bias, src/art/local/train.py:177-215 (a dense
+ *   [1,S,S] additive bias: 0 where  j <= i && (group[i] == group[j] ||
+ *   parent[i] == group[j]),  -inf elsewhere) and the masked softmax attention
+ *   of the model that consumes it as `causal_mask` (train.py:239-241; the
+ *   attention itself is third-party model code).  group_ids / parent_ids are
+ *   the PackedTensors rows of src/art/local/pack.py:13-21 (int64, pad -1).
+ *
+ * artk_attn_plan: once per packed row; the plan (device memory owned by the
+ *   caller, artk_attn_plan_bytes(S) bytes) is shared by every layer and head.
+ *   It holds int32 equality codes of the ids and, per block of queries, the
+ *   list of key blocks with at least one visible pair.
+ * artk_attn_fwd: out = softmax(scale * q k^T + bias) v, lse = log-sum-exp of
+ *   the biased scores (natural log).  Element (s, h, d) of q is at
+ *   q[s * q_stride_s + h * q_stride_h + d] (bf16; strides in elements,
+ *   multiples of 8), likewise k, v ([S, Hkv, D]) and out; query head h reads
+ *   key/value head h / (Hq / Hkv).  lse is f32 [Hq, S].
+ * artk_attn_bwd: dq, dk, dv (bf16, same addressing as q, k, v) from d_out.
+ * Requires S % 256 == 0, S <= 65536, D in {64, 128}.
+ * ------------------------------------------------------------------------- */
+size_t artk_attn_plan_bytes(int64_t S);
+int32_t artk_attn_plan(const int64_t* group_ids, const int64_t* parent_ids, int64_t S, void* plan,
+                       size_t plan_bytes, artk_stream_t stream);
+size_t artk_attn_fwd_workspace_bytes(int64_t S, int32_t Hkv, int32_t D);
+int32_t artk_attn_fwd(const void* q, const void* k, const void* v, const void* plan, int64_t S,
+                      int32_t Hq, int32_t Hkv, int32_t D, int64_t q_stride_s, int64_t q_stride_h,
+                      int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_s, int64_t v_stride_h,
+                      int64_t o_stride_s, int64_t o_stride_h, float scale, void* out, float* lse,
+                      void* workspace, size_t workspace_bytes, artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
  * artk_profile_enable(1) makes later calls bracket each dominant kernel with
  * HIP events on the launch stream; after the caller has synchronised,
@@ -224,6 +255,9 @@ int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_
 #define ARTK_PROF_SOFTMAX_GRAD 2
 #define ARTK_PROF_LORA_GEMM 3
 #define ARTK_PROF_MOE_GEMM 4
+#define ARTK_PROF_ATTN_FWD 5
+#define ARTK_PROF_ATTN_BWD_KV 6
+#define ARTK_PROF_ATTN_BWD_Q 7
 int32_t artk_profile_enable(int32_t on);
 int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches);
 
