@@ -27,6 +27,8 @@ constexpr int ATT_BM = 256;    // queries per work-group
 constexpr int ATT_BN = 64;     // keys per tile
 constexpr int ATT_STAGES = 3;
 constexpr int ATT_MAX_KB = 1024;  // key blocks per row the list in LDS can hold
+constexpr int ATT_BQ2 = 64;    // dK/dV kernel: queries per tile
+constexpr int ATT_BK2 = 128;   // dK/dV kernel: keys per work-group (4 waves x 32)
 
 // ----------------------------------------------------------------------------
 // Plan
@@ -133,10 +135,9 @@ struct AttnPlan {
   uint8_t* cls;        // [nQb][nKb]
   uint16_t* list;      // [nQb][nKb]
   int* cnt;            // [nQb]
-  int nQb2, nKb2;      // backward: query blocks of 64 / key blocks of 256 (see the backward kernels)
+  int nQb2, nKb2;      // dK/dV kernel: query tiles of 64 per key block of 128
   uint8_t* cls2;       // [nQb2][nKb2]
   uint8_t* cls2T;      // [nKb2][nQb2]
-  uint16_t* list_q;    // per query block (dQ kernel): reuses cls/list above
   uint16_t* list2T;    // [nKb2][nQb2] query blocks per key block
   int* cnt2T;          // [nKb2]
 };
@@ -145,8 +146,8 @@ static size_t attn_plan_layout(void* base, size_t bytes, int64_t S, AttnPlan& pl
   Workspace ws(base, bytes);
   pl.nQb = (int)(S / ATT_BM);
   pl.nKb = (int)(S / ATT_BN);
-  pl.nQb2 = (int)(S / ATT_BN);
-  pl.nKb2 = (int)(S / ATT_BM);
+  pl.nQb2 = (int)(S / ATT_BQ2);
+  pl.nKb2 = (int)(S / ATT_BK2);
   pl.gc = ws.take<int>((size_t)S);
   pl.pc = ws.take<int>((size_t)S);
   pl.cls = ws.take<uint8_t>((size_t)pl.nQb * pl.nKb);
@@ -156,7 +157,6 @@ static size_t attn_plan_layout(void* base, size_t bytes, int64_t S, AttnPlan& pl
   pl.cls2T = ws.take<uint8_t>((size_t)pl.nQb2 * pl.nKb2);
   pl.list2T = ws.take<uint16_t>((size_t)pl.nQb2 * pl.nKb2);
   pl.cnt2T = ws.take<int>((size_t)pl.nKb2);
-  pl.list_q = pl.list;
   return ws.ok() || base == nullptr ? ws.used : (size_t)-1;
 }
 
@@ -409,6 +409,443 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
 #undef ATTN_ISSUE
 }
 
+
+// ----------------------------------------------------------------------------
+// Backward
+//   P = exp(scale * S + bias - lse),  dV = P^T dO,  dP = dO V^T,
+//   dS = P o (dP - delta),  delta_i = sum_d dO[i,d] O[i,d],
+//   dQ = scale * dS K,  dK = scale * dS^T Q.
+// Two kernels, both free of atomics (bit-reproducible): one owns a block of
+// keys and accumulates dK, dV over the query tiles that see it (all query heads
+// of its key/value head), the other owns a block of queries and accumulates dQ
+// over its visible key tiles.  Each recomputes P from lse.
+// ----------------------------------------------------------------------------
+struct AttnBwdParams {
+  const uint16_t *Q, *K, *V, *dO;
+  const uint16_t *Kt, *Qt, *dOt;    // [H][D][S] transposed copies
+  const float* lse;                 // [Hq][S]
+  const float* delta;               // [Hq][S]
+  uint16_t *dQ, *dK, *dV;
+  int64_t q_ss, q_hs, k_ss, k_hs, v_ss, v_hs, do_ss, do_hs, dq_ss, dq_hs, dk_ss, dk_hs, dv_ss, dv_hs;
+  const int* gc;
+  const int* pc;
+  const uint16_t* list;    // per query block of 256: key tiles of 64
+  const int* cnt;
+  const uint16_t* listT;   // per key block of 128: query tiles of 64
+  const int* cntT;
+  int S, Hq, Hkv, nQb, nKb, nQb2, nKb2;
+  float scale, scale_log2e;
+};
+
+// delta[h][s] = sum_d dO[s,h,d] * O[s,h,d]; 16 lanes per (s, h).
+__global__ __launch_bounds__(256) void attn_delta_kernel(const uint16_t* __restrict__ O, int64_t o_ss,
+                                                         int64_t o_hs,
+                                                         const uint16_t* __restrict__ dO,
+                                                         int64_t do_ss, int64_t do_hs, int S, int H,
+                                                         int D, float* __restrict__ delta) {
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int sub = threadIdx.x & 15;
+  if (row >= (int64_t)S * H) return;
+  const int s = (int)(row / H), hh = (int)(row - (int64_t)s * H);
+  const uint16_t* op = O + (int64_t)s * o_ss + (int64_t)hh * o_hs;
+  const uint16_t* gp = dO + (int64_t)s * do_ss + (int64_t)hh * do_hs;
+  float acc = 0.f;
+  for (int d = sub * 8; d < D; d += 128) {
+    const bf16x8 a = *(const bf16x8*)(op + d);
+    const bf16x8 b = *(const bf16x8*)(gp + d);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
+  }
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (sub == 0) delta[(int64_t)hh * S + s] = acc;
+}
+
+// ---- dQ: 256 queries x one head per work-group, lane = query ----------------
+template <int D>
+struct AttnDqTile {
+  using F = AttnTile<D>;
+  static constexpr int V_OFF = F::K_BYTES;
+  static constexpr int KT_OFF = 2 * F::K_BYTES;
+  static constexpr int CODE_OFF = 2 * F::K_BYTES + F::V_BYTES;
+  static constexpr int STAGE = CODE_OFF + 1024;
+  static constexpr int N_PER = 2 * F::NK + F::NV + 1;
+};
+
+template <int D>
+__device__ __forceinline__ void attn_dq_issue(char* st, int kb, __amdgpu_buffer_rsrc_t rsrc_k,
+                                              __amdgpu_buffer_rsrc_t rsrc_v,
+                                              __amdgpu_buffer_rsrc_t rsrc_kt,
+                                              __amdgpu_buffer_rsrc_t rsrc_c,
+                                              const int (&voff_k)[AttnTile<D>::NK],
+                                              const int (&voff_v)[AttnTile<D>::NK],
+                                              const int (&voff_kt)[AttnTile<D>::NV], int64_t k_ss,
+                                              int64_t v_ss, int wave, int lane) {
+  using F = AttnTile<D>;
+  using T = AttnDqTile<D>;
+  const int k0 = kb * ATT_BN;
+#pragma unroll
+  for (int i = 0; i < F::NK; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_ptr_t)(st + (wave * F::NK + i) * 1024), 16,
+                                             voff_k[i], (int)(k0 * k_ss * 2), 0, 0);
+#pragma unroll
+  for (int i = 0; i < F::NK; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, (lds_ptr_t)(st + T::V_OFF + (wave * F::NK + i) * 1024),
+                                             16, voff_v[i], (int)(k0 * v_ss * 2), 0, 0);
+#pragma unroll
+  for (int i = 0; i < F::NV; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc_kt, (lds_ptr_t)(st + T::KT_OFF + (wave * F::NV + i) * 1024), 16, voff_kt[i], k0 * 2, 0, 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_c, (lds_ptr_t)(st + T::CODE_OFF), 4, lane * 4, k0 * 4, 0,
+                                           0);
+}
+
+template <int D>
+__global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
+  using F = AttnTile<D>;
+  using T = AttnDqTile<D>;
+  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * T::STAGE];
+  __shared__ uint16_t s_list[ATT_MAX_KB];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int hq = blockIdx.x % p.Hq;
+  const int qb = p.nQb - 1 - (int)(blockIdx.x / p.Hq);
+  const int hkv = hq / (p.Hq / p.Hkv);
+  const int q = qb * ATT_BM + wave * 32 + n;
+  const int cnt = p.cnt[qb];
+  for (int i = threadIdx.x; i < cnt; i += 512) s_list[i] = p.list[(int64_t)qb * p.nKb + i];
+
+  bf16x8 qf[D / 16], dof[D / 16];
+  {
+    const uint16_t* qp = p.Q + (int64_t)q * p.q_ss + (int64_t)hq * p.q_hs + 8 * h;
+    const uint16_t* gp = p.dO + (int64_t)q * p.do_ss + (int64_t)hq * p.do_hs + 8 * h;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      qf[s] = *(const bf16x8*)(qp + 16 * s);
+      dof[s] = *(const bf16x8*)(gp + 16 * s);
+    }
+  }
+  const int gi = p.gc[q], pi = p.pc[q];
+  const float nlse2 = -p.lse[(int64_t)hq * p.S + q] * LOG2E;
+  const float delta = p.delta[(int64_t)hq * p.S + q];
+
+  const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.K + (int64_t)hkv * p.k_hs), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.V + (int64_t)hkv * p.v_hs), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_kt = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.Kt + (int64_t)hkv * D * p.S), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_c =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.gc, 0, 0x7fffffff, 0x00020000);
+  int voff_k[F::NK], voff_v[F::NK], voff_kt[F::NV];
+#pragma unroll
+  for (int i = 0; i < F::NK; ++i) {
+    const int r = (wave * F::NK + i) * (64 / F::CHK) + lane / F::CHK;
+    const int c = (lane % F::CHK) ^ F::swz_k(r);
+    voff_k[i] = (int)(r * p.k_ss * 2) + c * 16;
+    voff_v[i] = (int)(r * p.v_ss * 2) + c * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < F::NV; ++i) {
+    const int r = (wave * F::NV + i) * 8 + lane / 8;
+    const int c = (lane % 8) ^ F::swz_v(r);
+    voff_kt[i] = r * p.S * 2 + c * 16;
+  }
+  __syncthreads();
+  auto* list_lds = s_list;
+#define ATTN_ISSUE(IT, STG)                                                                            \
+  attn_dq_issue<D>(smem + (STG) * T::STAGE, __builtin_amdgcn_readfirstlane(list_lds[IT] & 0x3fff),     \
+                   rsrc_k, rsrc_v, rsrc_kt, rsrc_c, voff_k, voff_v, voff_kt, p.k_ss, p.v_ss, wave, lane)
+
+  floatx16 dq[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) dq[dt][j] = 0.f;
+
+  if (cnt > 0) ATTN_ISSUE(0, 0);
+  if (cnt > 1) ATTN_ISSUE(1, 1);
+  int stage = 0;
+  for (int it = 0; it < cnt; ++it) {
+    if (it + 1 < cnt)
+      wait_vmcnt<T::N_PER>();
+    else
+      wait_vmcnt<0>();
+    __syncthreads();
+    if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
+    const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
+    const int kb = entry & 0x3fff;
+    const bool partial = (entry >> 14) == 1;
+    const char* st = smem + stage * T::STAGE;
+    const int* codes = (const int*)(st + T::CODE_OFF);
+
+    bf16x8 dsf[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      floatx16 sc, dp;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sc[j] = dp[j] = 0.f;
+      const int row = 32 * kt + n;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) {
+        const int off = row * (D * 2) + (((2 * s + h) ^ F::swz_k(row)) * 16);
+        const bf16x8 a = *(const bf16x8*)(st + off);
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[s], sc, 0, 0, 0);
+        const bf16x8 b = *(const bf16x8*)(st + T::V_OFF + off);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, dof[s], dp, 0, 0, 0);
+      }
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int kk = 32 * kt + 8 * g4 + 4 * h;
+        int kcv[4] = {0, 0, 0, 0};
+        if (partial) {
+          const int4 kc = *(const int4*)(codes + kk);
+          kcv[0] = kc.x; kcv[1] = kc.y; kcv[2] = kc.z; kcv[3] = kc.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = 4 * g4 + e;
+          float x = __builtin_fmaf(sc[j], p.scale_log2e, nlse2);
+          if (partial && !attn_visible(q, kb * ATT_BN + kk + e, gi, pi, kcv[e])) x = -INFINITY;
+          const float pr = __builtin_amdgcn_exp2f(x);
+          dsf[2 * kt + j / 8][j % 8] = (__bf16)(pr * (dp[j] - delta));
+        }
+      }
+    }
+    const char* kt_tile = st + T::KT_OFF;
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt) {
+        const int row = 32 * dt + n;
+        const int sw = F::swz_v(row);
+        const bf16x4 lo = *(const bf16x4*)(kt_tile + row * 128 + (((2 * s2) ^ sw) * 16) + 8 * h);
+        const bf16x4 hi = *(const bf16x4*)(kt_tile + row * 128 + (((2 * s2 + 1) ^ sw) * 16) + 8 * h);
+        const bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, dsf[s2], dq[dt], 0, 0, 0);
+      }
+    }
+    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
+  }
+#undef ATTN_ISSUE
+  uint16_t* op = p.dQ + (int64_t)q * p.dq_ss + (int64_t)hq * p.dq_hs + 4 * h;
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (__bf16)(dq[dt][4 * g4 + e] * p.scale);
+      *(bf16x4*)(op + 32 * dt + 8 * g4) = v;
+    }
+}
+
+// ---- dK, dV: 128 keys x one key/value head per work-group, lane = key --------
+template <int D>
+struct AttnKvTile {
+  using F = AttnTile<D>;
+  static constexpr int Q_BYTES = ATT_BQ2 * D * 2;       // [query][d] tiles (Q, dO)
+  static constexpr int T_BYTES = D * ATT_BQ2 * 2;       // [d][query] tiles (Q^T, dO^T)
+  static constexpr int DO_OFF = Q_BYTES;
+  static constexpr int QT_OFF = 2 * Q_BYTES;
+  static constexpr int DOT_OFF = 2 * Q_BYTES + T_BYTES;
+  static constexpr int ROW_OFF = 2 * Q_BYTES + 2 * T_BYTES;  // lse, delta, gc, pc of the 64 queries
+  static constexpr int STAGE = ROW_OFF + 1024;
+  static constexpr int NQ = Q_BYTES / 1024 / 4;         // DMA instructions per wave (4 waves)
+  static constexpr int NT = T_BYTES / 1024 / 4;
+  static constexpr int N_PER = 2 * NQ + 2 * NT + 1;
+};
+
+// DMA of one (query head, query tile) into an LDS stage of the dK/dV kernel: this
+// wave's share of the Q, dO, Q^T and dO^T tiles, and one of the four per-query
+// arrays (wave 0: lse, 1: delta, 2: group codes, 3: parent codes).
+template <int D>
+__device__ __forceinline__ void attn_kv_issue(
+    char* st, int hq, int q0, __amdgpu_buffer_rsrc_t rsrc_q, __amdgpu_buffer_rsrc_t rsrc_do,
+    __amdgpu_buffer_rsrc_t rsrc_qt, __amdgpu_buffer_rsrc_t rsrc_dot, __amdgpu_buffer_rsrc_t rsrc_row,
+    const int (&voff_q)[AttnKvTile<D>::NQ], const int (&voff_do)[AttnKvTile<D>::NQ],
+    const int (&voff_t)[AttnKvTile<D>::NT], const AttnBwdParams& p, int wave, int lane) {
+  using T = AttnKvTile<D>;
+  const int so_q = (int)((q0 * p.q_ss + hq * p.q_hs) * 2);
+  const int so_do = (int)((q0 * p.do_ss + hq * p.do_hs) * 2);
+  const int so_t = (int)(((int64_t)hq * D * p.S + q0) * 2);
+#pragma unroll
+  for (int i = 0; i < T::NQ; ++i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, (lds_ptr_t)(st + (wave * T::NQ + i) * 1024), 16,
+                                             voff_q[i], so_q, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_do, (lds_ptr_t)(st + T::DO_OFF + (wave * T::NQ + i) * 1024),
+                                             16, voff_do[i], so_do, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < T::NT; ++i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_qt, (lds_ptr_t)(st + T::QT_OFF + (wave * T::NT + i) * 1024),
+                                             16, voff_t[i], so_t, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_dot, (lds_ptr_t)(st + T::DOT_OFF + (wave * T::NT + i) * 1024),
+                                             16, voff_t[i], so_t, 0, 0);
+  }
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row, (lds_ptr_t)(st + T::ROW_OFF + wave * 256), 4, lane * 4,
+                                           (int)(((wave < 2 ? (int64_t)hq * p.S : 0) + q0) * 4), 0, 0);
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
+  using F = AttnTile<D>;
+  using T = AttnKvTile<D>;
+  __shared__ __attribute__((aligned(1024))) char smem[2 * T::STAGE];
+  __shared__ uint16_t s_list[ATT_MAX_KB];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int hkv = blockIdx.x % p.Hkv;
+  const int kb = (int)(blockIdx.x / p.Hkv);  // early key blocks are seen by the most queries
+  const int rep = p.Hq / p.Hkv;
+  const int key = kb * ATT_BK2 + wave * 32 + n;
+  const int cntT = p.cntT[kb];
+  for (int i = threadIdx.x; i < cntT; i += 256) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
+
+  bf16x8 kf[D / 16], vf[D / 16];
+  {
+    const uint16_t* kp = p.K + (int64_t)key * p.k_ss + (int64_t)hkv * p.k_hs + 8 * h;
+    const uint16_t* vp = p.V + (int64_t)key * p.v_ss + (int64_t)hkv * p.v_hs + 8 * h;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      kf[s] = *(const bf16x8*)(kp + 16 * s);
+      vf[s] = *(const bf16x8*)(vp + 16 * s);
+    }
+  }
+  const int gk = p.gc[key];
+
+  const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc((void*)p.Q, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_do = __builtin_amdgcn_make_buffer_rsrc((void*)p.dO, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_qt = __builtin_amdgcn_make_buffer_rsrc((void*)p.Qt, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_dot = __builtin_amdgcn_make_buffer_rsrc((void*)p.dOt, 0, 0x7fffffff, 0x00020000);
+  // wave w brings in one of the four per-query arrays
+  const void* row_src = wave == 0 ? (const void*)p.lse : wave == 1 ? (const void*)p.delta
+                        : wave == 2 ? (const void*)p.gc : (const void*)p.pc;
+  const __amdgpu_buffer_rsrc_t rsrc_row = __builtin_amdgcn_make_buffer_rsrc((void*)row_src, 0, 0x7fffffff, 0x00020000);
+  int voff_q[T::NQ], voff_do[T::NQ], voff_t[T::NT];
+#pragma unroll
+  for (int i = 0; i < T::NQ; ++i) {
+    const int r = (wave * T::NQ + i) * (64 / F::CHK) + lane / F::CHK;
+    const int c = (lane % F::CHK) ^ F::swz_k(r);
+    voff_q[i] = (int)(r * p.q_ss * 2) + c * 16;
+    voff_do[i] = (int)(r * p.do_ss * 2) + c * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < T::NT; ++i) {
+    const int r = (wave * T::NT + i) * 8 + lane / 8;
+    const int c = (lane % 8) ^ F::swz_v(r);
+    voff_t[i] = r * p.S * 2 + c * 16;
+  }
+  __syncthreads();
+
+  auto* list_lds = s_list;
+  // tile `IT` of the flattened (head of the group, visible query tile) sequence
+#define ATTN_ISSUE(IT, STG)                                                                          \
+  do {                                                                                               \
+    const int hi_ = (IT) / cntT, ti_ = (IT) - hi_ * cntT;                                             \
+    attn_kv_issue<D>(smem + (STG) * T::STAGE, hkv * rep + hi_,                                        \
+                     __builtin_amdgcn_readfirstlane(list_lds[ti_] & 0x3fff) * ATT_BQ2, rsrc_q, rsrc_do, \
+                     rsrc_qt, rsrc_dot, rsrc_row, voff_q, voff_do, voff_t, p, wave, lane);            \
+  } while (0)
+
+  floatx16 dk[D / 32], dv[D / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) dk[dt][j] = dv[dt][j] = 0.f;
+
+  const int total = cntT * rep;
+  if (total > 0) ATTN_ISSUE(0, 0);
+  int ti = 0;
+  for (int it = 0; it < total; ++it) {
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (it + 1 < total) ATTN_ISSUE(it + 1, (it + 1) & 1);
+    const int entry = __builtin_amdgcn_readfirstlane(s_list[ti]);
+    ti = ti + 1 == cntT ? 0 : ti + 1;
+    const int q0 = (entry & 0x3fff) * ATT_BQ2;
+    const bool partial = (entry >> 14) == 1;
+    const char* st = smem + (it & 1) * T::STAGE;
+    const float* r_lse = (const float*)(st + T::ROW_OFF);
+    const float* r_delta = r_lse + 64;
+    const int* r_gc = (const int*)(r_lse + 128);
+    const int* r_pc = r_gc + 64;
+
+    bf16x8 pf[4], dsf[4];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      floatx16 sc, dp;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sc[j] = dp[j] = 0.f;
+      const int row = 32 * qt + n;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) {
+        const int off = row * (D * 2) + (((2 * s + h) ^ F::swz_k(row)) * 16);
+        const bf16x8 a = *(const bf16x8*)(st + off);
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, kf[s], sc, 0, 0, 0);
+        const bf16x8 b = *(const bf16x8*)(st + T::DO_OFF + off);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, vf[s], dp, 0, 0, 0);
+      }
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int qi = 32 * qt + 8 * g4 + 4 * h;
+        const floatx4 l4 = *(const floatx4*)(r_lse + qi);
+        const floatx4 d4 = *(const floatx4*)(r_delta + qi);
+        int gq[4] = {0, 0, 0, 0}, pq[4] = {0, 0, 0, 0};
+        if (partial) {
+          const int4 a4 = *(const int4*)(r_gc + qi);
+          const int4 b4 = *(const int4*)(r_pc + qi);
+          gq[0] = a4.x; gq[1] = a4.y; gq[2] = a4.z; gq[3] = a4.w;
+          pq[0] = b4.x; pq[1] = b4.y; pq[2] = b4.z; pq[3] = b4.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = 4 * g4 + e;
+          float x = __builtin_fmaf(sc[j], p.scale_log2e, -l4[e] * LOG2E);
+          if (partial && !attn_visible(q0 + qi + e, key, gq[e], pq[e], gk)) x = -INFINITY;
+          const float pr = __builtin_amdgcn_exp2f(x);
+          pf[2 * qt + j / 8][j % 8] = (__bf16)pr;
+          dsf[2 * qt + j / 8][j % 8] = (__bf16)(pr * (dp[j] - d4[e]));
+        }
+      }
+    }
+    const char* qt_tile = st + T::QT_OFF;
+    const char* dot_tile = st + T::DOT_OFF;
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt) {
+        const int row = 32 * dt + n;
+        const int sw = F::swz_v(row);
+        const int o_lo = row * 128 + (((2 * s2) ^ sw) * 16) + 8 * h;
+        const int o_hi = row * 128 + (((2 * s2 + 1) ^ sw) * 16) + 8 * h;
+        const bf16x8 a = __builtin_shufflevector(*(const bf16x4*)(dot_tile + o_lo),
+                                                 *(const bf16x4*)(dot_tile + o_hi), 0, 1, 2, 3, 4, 5, 6, 7);
+        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[s2], dv[dt], 0, 0, 0);
+        const bf16x8 b = __builtin_shufflevector(*(const bf16x4*)(qt_tile + o_lo),
+                                                 *(const bf16x4*)(qt_tile + o_hi), 0, 1, 2, 3, 4, 5, 6, 7);
+        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, dsf[s2], dk[dt], 0, 0, 0);
+      }
+    }
+  }
+#undef ATTN_ISSUE
+  uint16_t* kp = p.dK + (int64_t)key * p.dk_ss + (int64_t)hkv * p.dk_hs + 4 * h;
+  uint16_t* vp = p.dV + (int64_t)key * p.dv_ss + (int64_t)hkv * p.dv_hs + 4 * h;
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; ++g4) {
+      bf16x4 a, b;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        a[e] = (__bf16)(dk[dt][4 * g4 + e] * p.scale);
+        b[e] = (__bf16)dv[dt][4 * g4 + e];
+      }
+      *(bf16x4*)(kp + 32 * dt + 8 * g4) = a;
+      *(bf16x4*)(vp + 32 * dt + 8 * g4) = b;
+    }
+}
+
 }  // namespace artk
 
 using namespace artk;
@@ -443,7 +880,7 @@ int32_t artk_attn_plan(const int64_t* group_ids, const int64_t* parent_ids, int6
   attn_compact_kernel<<<(unsigned)pl.nQb, 256, 0, st>>>(pl.cls, pl.nKb, pl.list, pl.cnt);
   ARTK_CHECK_LAUNCH();
   attn_classify_kernel<<<dim3((unsigned)((pl.nKb2 + 3) / 4), (unsigned)pl.nQb2), 256, 0, st>>>(
-      pl.gc, pl.pc, ATT_BN, ATT_BM, pl.nQb2, pl.nKb2, pl.cls2, pl.cls2T);
+      pl.gc, pl.pc, ATT_BQ2, ATT_BK2, pl.nQb2, pl.nKb2, pl.cls2, pl.cls2T);
   ARTK_CHECK_LAUNCH();
   attn_compact_kernel<<<(unsigned)pl.nKb2, 256, 0, st>>>(pl.cls2T, pl.nQb2, pl.list2T, pl.cnt2T);
   ARTK_CHECK_LAUNCH();
@@ -532,6 +969,109 @@ int32_t artk_attn_fwd(const void* q, const void* k, const void* v, const void* p
   else
     attn_fwd_kernel<64><<<grid, 512, 0, st>>>(p);
   prof_end(PROF_ATTN_FWD, st);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+size_t artk_attn_bwd_workspace_bytes(int64_t S, int32_t Hq, int32_t Hkv, int32_t D) {
+  Workspace ws(nullptr, 0);
+  ws.take<uint16_t>((size_t)S * Hkv * D);
+  ws.take<uint16_t>((size_t)S * Hq * D);
+  ws.take<uint16_t>((size_t)S * Hq * D);
+  ws.take<float>((size_t)S * Hq);
+  return ws.used + 256;
+}
+
+int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                      const void* d_out, const void* plan, int64_t S, int32_t Hq, int32_t Hkv,
+                      int32_t D, const int64_t* strides, float scale, void* dq, void* dk, void* dv,
+                      void* workspace, size_t workspace_bytes, artk_stream_t stream) {
+  ARTK_CHECK_ARG(q && k && v && out && lse && d_out && plan && strides && dq && dk && dv,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) && aligned16(d_out) &&
+                     aligned16(dq) && aligned16(dk) && aligned16(dv),
+                 "tensors must be 16-byte aligned");
+  int32_t rc = attn_check(S, Hq, Hkv, D, strides, 16);
+  if (rc) return rc;
+  // the dK/dV kernel addresses q and d_out by head through 31-bit offsets
+  ARTK_CHECK_ARG((S * strides[0] + Hq * strides[1]) * 2 < (1ll << 31) &&
+                     (S * strides[8] + Hq * strides[9]) * 2 < (1ll << 31) &&
+                     (int64_t)S * Hq * D * 2 < (1ll << 31),
+                 "q / d_out span 2 GiB or more");
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* kt = ws.take<uint16_t>((size_t)S * Hkv * D);
+  uint16_t* qt = ws.take<uint16_t>((size_t)S * Hq * D);
+  uint16_t* dot = ws.take<uint16_t>((size_t)S * Hq * D);
+  float* delta = ws.take<float>((size_t)S * Hq);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  AttnPlan pl;
+  attn_plan_layout(const_cast<void*>(plan), (size_t)1 << 40, S, pl);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 tb((unsigned)(S / 64), (unsigned)(D / 64), 1);
+  attn_transpose_kernel<<<dim3(tb.x, tb.y, (unsigned)Hkv), 256, 0, st>>>((const uint16_t*)k, strides[2],
+                                                                        strides[3], (int)S, D, kt);
+  ARTK_CHECK_LAUNCH();
+  attn_transpose_kernel<<<dim3(tb.x, tb.y, (unsigned)Hq), 256, 0, st>>>((const uint16_t*)q, strides[0],
+                                                                       strides[1], (int)S, D, qt);
+  ARTK_CHECK_LAUNCH();
+  attn_transpose_kernel<<<dim3(tb.x, tb.y, (unsigned)Hq), 256, 0, st>>>((const uint16_t*)d_out, strides[8],
+                                                                       strides[9], (int)S, D, dot);
+  ARTK_CHECK_LAUNCH();
+  attn_delta_kernel<<<(unsigned)((S * Hq + 15) / 16), 256, 0, st>>>(
+      (const uint16_t*)out, strides[6], strides[7], (const uint16_t*)d_out, strides[8], strides[9], (int)S,
+      Hq, D, delta);
+  ARTK_CHECK_LAUNCH();
+  AttnBwdParams p;
+  p.Q = (const uint16_t*)q;
+  p.K = (const uint16_t*)k;
+  p.V = (const uint16_t*)v;
+  p.dO = (const uint16_t*)d_out;
+  p.Kt = kt;
+  p.Qt = qt;
+  p.dOt = dot;
+  p.lse = lse;
+  p.delta = delta;
+  p.dQ = (uint16_t*)dq;
+  p.dK = (uint16_t*)dk;
+  p.dV = (uint16_t*)dv;
+  p.q_ss = strides[0];  p.q_hs = strides[1];
+  p.k_ss = strides[2];  p.k_hs = strides[3];
+  p.v_ss = strides[4];  p.v_hs = strides[5];
+  p.do_ss = strides[8]; p.do_hs = strides[9];
+  p.dq_ss = strides[10]; p.dq_hs = strides[11];
+  p.dk_ss = strides[12]; p.dk_hs = strides[13];
+  p.dv_ss = strides[14]; p.dv_hs = strides[15];
+  p.gc = pl.gc;
+  p.pc = pl.pc;
+  p.list = pl.list;
+  p.cnt = pl.cnt;
+  p.listT = pl.list2T;
+  p.cntT = pl.cnt2T;
+  p.S = (int)S;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.nQb = pl.nQb;
+  p.nKb = pl.nKb;
+  p.nQb2 = pl.nQb2;
+  p.nKb2 = pl.nKb2;
+  p.scale = scale;
+  p.scale_log2e = scale * LOG2E;
+  prof_begin(PROF_ATTN_BWD_KV, st);
+  if (D == 128)
+    attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hkv), 256, 0, st>>>(p);
+  else
+    attn_bwd_kv_kernel<64><<<(unsigned)(pl.nKb2 * Hkv), 256, 0, st>>>(p);
+  prof_end(PROF_ATTN_BWD_KV, st);
+  ARTK_CHECK_LAUNCH();
+  prof_begin(PROF_ATTN_BWD_Q, st);
+  if (D == 128)
+    attn_bwd_dq_kernel<128><<<(unsigned)(pl.nQb * Hq), 512, 0, st>>>(p);
+  else
+    attn_bwd_dq_kernel<64><<<(unsigned)(pl.nQb * Hq), 512, 0, st>>>(p);
+  prof_end(PROF_ATTN_BWD_Q, st);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

@@ -432,6 +432,33 @@ def attn_fwd(q, k, v, plan: AttnPlan, scale: Optional[float] = None):
     return out, lse
 
 
+def attn_bwd(q, k, v, out, lse, d_out, plan: AttnPlan, scale: Optional[float] = None):
+    """(dq, dk, dv) bf16, contiguous [S, H, D], for the upstream gradient d_out of attn_fwd's out."""
+    import ctypes as C
+
+    S, Hq, D = q.shape
+    Hkv = k.shape[1]
+    lib = _lib.load()
+    dev = q.device
+    dq = torch.empty((S, Hq, D), dtype=torch.bfloat16, device=dev)
+    dk = torch.empty((S, Hkv, D), dtype=torch.bfloat16, device=dev)
+    dv = torch.empty((S, Hkv, D), dtype=torch.bfloat16, device=dev)
+    _need(lse, "lse", torch.float32, (Hq, S))
+    strides = []
+    for name, t in (("q", q), ("k", k), ("v", v), ("out", out), ("d_out", d_out), ("dq", dq), ("dk", dk),
+                    ("dv", dv)):
+        strides += list(_shd(t, name))
+    arr = (C.c_int64 * 16)(*strides)
+    ws = _workspace(lib.artk_attn_bwd_workspace_bytes(S, Hq, Hkv, D), dev)
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    _lib.check(
+        lib.artk_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                          d_out.data_ptr(), plan.buf.data_ptr(), S, Hq, Hkv, D, arr, scale, dq.data_ptr(),
+                          dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), ws.numel(), _stream(dev))
+    )
+    return dq, dk, dv
+
+
 # -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------

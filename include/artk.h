@@ -242,6 +242,12 @@ int32_t artk_attn_fwd(const void* q, const void* k, const void* v, const void* p
                       int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_s, int64_t v_stride_h,
                       int64_t o_stride_s, int64_t o_stride_h, float scale, void* out, float* lse,
                       void* workspace, size_t workspace_bytes, artk_stream_t stream);
+/* strides: 16 element strides, (stride_s, stride_h) of q, k, v, out, d_out, dq, dk, dv in that order. */
+size_t artk_attn_bwd_workspace_bytes(int64_t S, int32_t Hq, int32_t Hkv, int32_t D);
+int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                      const void* d_out, const void* plan, int64_t S, int32_t Hq, int32_t Hkv,
+                      int32_t D, const int64_t* strides, float scale, void* dq, void* dk, void* dv,
+                      void* workspace, size_t workspace_bytes, artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).

@@ -81,3 +81,42 @@ def test_attn_fwd_head_major_layout_and_random_ids(artk_lib, gpu):
     out, lse = ops.attn_fwd(hm(q), hm(k), hm(v), plan)
     assert (lse.cpu() - ref_lse).abs().max().item() <= 2e-3
     assert rel_l2(out.float().cpu(), ref_out) <= 1e-2
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("Hq,Hkv,D", [(4, 2, 128), (2, 2, 64), (7, 1, 128)])
+def test_attn_bwd_matches_oracle(artk_lib, gpu, layout, Hq, Hkv, D):
+    S, npr, pl, nc, cl = LAYOUTS[layout]
+    print(f"attn bwd {layout} Hq={Hq} Hkv={Hkv} D={D}", flush=True)
+    q, k, v = make_qkv(S + Hq + D + 1, S, Hq, Hkv, D)
+    g = torch.Generator().manual_seed(S + 5)
+    d_out = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16)
+    group, parent = synthetic.packed_row_ids(S + 1, S, npr, pl, nc, cl)
+    _, ref_dq, ref_dk, ref_dv = attn_oracle.attention_grads(q, k, v, group, parent, d_out)
+    plan = ops.attn_plan(group.to(gpu), parent.to(gpu))
+    qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.attn_fwd(qd, kd, vd, plan)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, out, lse, d_out.to(gpu), plan)
+    assert rel_l2(dv.float().cpu(), ref_dv) <= 1e-2
+    assert rel_l2(dq.float().cpu(), ref_dq) <= 1e-2
+    assert rel_l2(dk.float().cpu(), ref_dk) <= 1e-2
+    # run-to-run determinism (no atomics)
+    dq2, dk2, dv2 = ops.attn_bwd(qd, kd, vd, out, lse, d_out.to(gpu), plan)
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
+def test_attn_bwd_random_ids(artk_lib, gpu):
+    S, Hq, Hkv, D = 512, 4, 2, 128
+    q, k, v = make_qkv(21, S, Hq, Hkv, D)
+    g = torch.Generator().manual_seed(22)
+    d_out = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16)
+    group = torch.randint(0, 5, (S,), generator=g)
+    parent = torch.randint(0, 5, (S,), generator=g)
+    _, ref_dq, ref_dk, ref_dv = attn_oracle.attention_grads(q, k, v, group, parent, d_out)
+    plan = ops.attn_plan(group.to(gpu), parent.to(gpu))
+    qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.attn_fwd(qd, kd, vd, plan)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, out, lse, d_out.to(gpu), plan)
+    assert rel_l2(dq.float().cpu(), ref_dq) <= 1e-2
+    assert rel_l2(dk.float().cpu(), ref_dk) <= 1e-2
+    assert rel_l2(dv.float().cpu(), ref_dv) <= 1e-2
