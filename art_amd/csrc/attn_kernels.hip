@@ -426,6 +426,7 @@ struct AttnBwdParams {
   const float* lse;                 // [Hq][S]
   const float* delta;               // [Hq][S]
   uint16_t *dQ, *dK, *dV;
+  float *pK, *pV;                   // [Hq/Hkv][S][Hkv][D] per-head partial sums (grouped-query heads only)
   int64_t q_ss, q_hs, k_ss, k_hs, v_ss, v_hs, do_ss, do_hs, dq_ss, dq_hs, dk_ss, dk_hs, dv_ss, dv_hs;
   const int* gc;
   const int* pc;
@@ -640,7 +641,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
     }
 }
 
-// ---- dK, dV: 128 keys x one key/value head per work-group, lane = key --------
+// ---- dK, dV: 128 keys x one query head per work-group, lane = key ------------
+// With grouped-query heads the work-groups of the heads that share a key/value
+// head write fp32 partial sums, which attn_kv_reduce_kernel adds in a fixed order.
 template <int D>
 struct AttnKvTile {
   using F = AttnTile<D>;
@@ -695,9 +698,10 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
   __shared__ uint16_t s_list[ATT_MAX_KB];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, h = lane >> 5;
-  const int hkv = blockIdx.x % p.Hkv;
-  const int kb = (int)(blockIdx.x / p.Hkv);  // early key blocks are seen by the most queries
+  const int hq = blockIdx.x % p.Hq;
+  const int kb = (int)(blockIdx.x / p.Hq);  // early key blocks are seen by the most queries
   const int rep = p.Hq / p.Hkv;
+  const int hkv = hq / rep;
   const int key = kb * ATT_BK2 + wave * 32 + n;
   const int cntT = p.cntT[kb];
   for (int i = threadIdx.x; i < cntT; i += 256) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
@@ -739,14 +743,10 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
   __syncthreads();
 
   auto* list_lds = s_list;
-  // tile `IT` of the flattened (head of the group, visible query tile) sequence
 #define ATTN_ISSUE(IT, STG)                                                                          \
-  do {                                                                                               \
-    const int hi_ = (IT) / cntT, ti_ = (IT) - hi_ * cntT;                                             \
-    attn_kv_issue<D>(smem + (STG) * T::STAGE, hkv * rep + hi_,                                        \
-                     __builtin_amdgcn_readfirstlane(list_lds[ti_] & 0x3fff) * ATT_BQ2, rsrc_q, rsrc_do, \
-                     rsrc_qt, rsrc_dot, rsrc_row, voff_q, voff_do, voff_t, p, wave, lane);            \
-  } while (0)
+  attn_kv_issue<D>(smem + (STG) * T::STAGE, hq,                                                       \
+                   __builtin_amdgcn_readfirstlane(list_lds[IT] & 0x3fff) * ATT_BQ2, rsrc_q, rsrc_do,  \
+                   rsrc_qt, rsrc_dot, rsrc_row, voff_q, voff_do, voff_t, p, wave, lane)
 
   floatx16 dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -754,15 +754,13 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) dk[dt][j] = dv[dt][j] = 0.f;
 
-  const int total = cntT * rep;
+  const int total = cntT;
   if (total > 0) ATTN_ISSUE(0, 0);
-  int ti = 0;
   for (int it = 0; it < total; ++it) {
     wait_vmcnt<0>();
     __syncthreads();
     if (it + 1 < total) ATTN_ISSUE(it + 1, (it + 1) & 1);
-    const int entry = __builtin_amdgcn_readfirstlane(s_list[ti]);
-    ti = ti + 1 == cntT ? 0 : ti + 1;
+    const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int q0 = (entry & 0x3fff) * ATT_BQ2;
     const bool partial = (entry >> 14) == 1;
     const char* st = smem + (it & 1) * T::STAGE;
@@ -829,6 +827,23 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
     }
   }
 #undef ATTN_ISSUE
+  if (rep > 1) {
+    const int64_t o = ((((int64_t)(hq - hkv * rep) * p.S + key) * p.Hkv + hkv) * D) + 4 * h;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        floatx4 a, b;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = dk[dt][4 * g4 + e];
+          b[e] = dv[dt][4 * g4 + e];
+        }
+        *(floatx4*)(p.pK + o + 32 * dt + 8 * g4) = a;
+        *(floatx4*)(p.pV + o + 32 * dt + 8 * g4) = b;
+      }
+    return;
+  }
   uint16_t* kp = p.dK + (int64_t)key * p.dk_ss + (int64_t)hkv * p.dk_hs + 4 * h;
   uint16_t* vp = p.dV + (int64_t)key * p.dv_ss + (int64_t)hkv * p.dv_hs + 4 * h;
 #pragma unroll
@@ -844,6 +859,36 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
       *(bf16x4*)(kp + 32 * dt + 8 * g4) = a;
       *(bf16x4*)(vp + 32 * dt + 8 * g4) = b;
     }
+}
+
+// dK = scale * sum_r pK[r], dV = sum_r pV[r] over the query heads r of a group, in
+// index order; 4 elements per thread.
+__global__ __launch_bounds__(256) void attn_kv_reduce_kernel(const float* __restrict__ pK,
+                                                             const float* __restrict__ pV, int rep,
+                                                             int64_t S, int Hkv, int D, float scale,
+                                                             uint16_t* __restrict__ dK, int64_t dk_ss,
+                                                             int64_t dk_hs, uint16_t* __restrict__ dV,
+                                                             int64_t dv_ss, int64_t dv_hs) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int d4 = D / 4;
+  const int64_t n = S * Hkv * d4;
+  if (i >= n) return;
+  const int c = (int)(i % d4);
+  const int hh = (int)((i / d4) % Hkv);
+  const int64_t s = i / ((int64_t)d4 * Hkv);
+  floatx4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < rep; ++r) {
+    a += ((const floatx4*)pK)[(int64_t)r * n + i];
+    b += ((const floatx4*)pV)[(int64_t)r * n + i];
+  }
+  bf16x4 oa, ob;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    oa[e] = (__bf16)(a[e] * scale);
+    ob[e] = (__bf16)b[e];
+  }
+  *(bf16x4*)(dK + s * dk_ss + (int64_t)hh * dk_hs + 4 * c) = oa;
+  *(bf16x4*)(dV + s * dv_ss + (int64_t)hh * dv_hs + 4 * c) = ob;
 }
 
 }  // namespace artk
@@ -979,6 +1024,10 @@ size_t artk_attn_bwd_workspace_bytes(int64_t S, int32_t Hq, int32_t Hkv, int32_t
   ws.take<uint16_t>((size_t)S * Hq * D);
   ws.take<uint16_t>((size_t)S * Hq * D);
   ws.take<float>((size_t)S * Hq);
+  if (Hq != Hkv) {
+    ws.take<float>((size_t)S * Hq * D);
+    ws.take<float>((size_t)S * Hq * D);
+  }
   return ws.used + 256;
 }
 
@@ -1003,6 +1052,11 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   uint16_t* qt = ws.take<uint16_t>((size_t)S * Hq * D);
   uint16_t* dot = ws.take<uint16_t>((size_t)S * Hq * D);
   float* delta = ws.take<float>((size_t)S * Hq);
+  float *pk = nullptr, *pv = nullptr;
+  if (Hq != Hkv) {
+    pk = ws.take<float>((size_t)S * Hq * D);
+    pv = ws.take<float>((size_t)S * Hq * D);
+  }
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
@@ -1037,6 +1091,8 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   p.dQ = (uint16_t*)dq;
   p.dK = (uint16_t*)dk;
   p.dV = (uint16_t*)dv;
+  p.pK = pk;
+  p.pV = pv;
   p.q_ss = strides[0];  p.q_hs = strides[1];
   p.k_ss = strides[2];  p.k_hs = strides[3];
   p.v_ss = strides[4];  p.v_hs = strides[5];
@@ -1061,11 +1117,18 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   p.scale_log2e = scale * LOG2E;
   prof_begin(PROF_ATTN_BWD_KV, st);
   if (D == 128)
-    attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hkv), 256, 0, st>>>(p);
+    attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hq), 256, 0, st>>>(p);
   else
-    attn_bwd_kv_kernel<64><<<(unsigned)(pl.nKb2 * Hkv), 256, 0, st>>>(p);
+    attn_bwd_kv_kernel<64><<<(unsigned)(pl.nKb2 * Hq), 256, 0, st>>>(p);
   prof_end(PROF_ATTN_BWD_KV, st);
   ARTK_CHECK_LAUNCH();
+  if (Hq != Hkv) {
+    const int64_t n4 = S * Hkv * (D / 4);
+    attn_kv_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(
+        pk, pv, Hq / Hkv, S, Hkv, D, scale, (uint16_t*)dk, strides[12], strides[13], (uint16_t*)dv,
+        strides[14], strides[15]);
+    ARTK_CHECK_LAUNCH();
+  }
   prof_begin(PROF_ATTN_BWD_Q, st);
   if (D == 128)
     attn_bwd_dq_kernel<128><<<(unsigned)(pl.nQb * Hq), 512, 0, st>>>(p);
