@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe", "attn"],
                     help="c3 (default, the headline): fused GRPO step at the Qwen2.5-7B shape; c1/c4: the "
                          "0.5B / 14B shapes; lora: LoRA linear fwd+bwd at the Qwen2.5-3B shapes; moe: "
                          "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
@@ -239,6 +239,87 @@ def bench_moe(args):
     print(json.dumps(res))
 
 
+def bench_attn(args):
+    """Packed-row attention of one layer at the Qwen2.5-7B head shape: a row of 16384 positions
+    holding 8 prompts of 128 tokens, each with 4 completions of 480 tokens (the packer's layout),
+    28 query / 4 key-value heads of 128.  One step = plan reuse + forward + backward; value =
+    algorithmic TFLOP/s over the visible (query, key) pairs: 4 N D Hq forward + 10 N D Hq backward."""
+    import torch
+
+    from art_amd import ops, synthetic
+
+    dev = torch.device("cuda:0")
+    S, Hq, Hkv, D = 16384, 28, 4, 128
+    layout = (8, 128, 4, 480)
+    g = torch.Generator().manual_seed(1006)
+    q = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16).to(dev)
+    k = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16).to(dev)
+    d_out = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16).to(dev)
+    group, parent = synthetic.packed_row_ids(1006, S, *layout)
+    # visible pairs from the layout: a prompt token sees its prompt prefix, a completion token its
+    # prompt and its completion prefix, a padding token the padding before it
+    npr, pl, nc, cl = layout
+    pad = S - npr * (pl + nc * cl)
+    n_vis = npr * (pl * (pl + 1) // 2 + nc * (cl * pl + cl * (cl + 1) // 2)) + pad * (pad + 1) // 2
+    plan = ops.attn_plan(group.to(dev), parent.to(dev))
+    state = {}
+
+    def step():
+        out, lse = ops.attn_fwd(q, k, v, plan)
+        state["grads"] = ops.attn_bwd(q, k, v, out, lse, d_out, plan)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    prof = {name: ops.profile_collect(kind) for name, kind in
+            (("attn_fwd_kernel", ops.PROF_ATTN_FWD), ("attn_bwd_kv_kernel", ops.PROF_ATTN_BWD_KV),
+             ("attn_bwd_dq_kernel", ops.PROF_ATTN_BWD_Q))}
+    ops.profile_enable(False)
+    unit_flops = 2.0 * n_vis * D * Hq           # one product over the visible pairs
+    flops = 14.0 * n_vis * D * Hq
+    res = base_result(args, "packed-row attention fwd+bwd TFLOP/s over visible pairs (7B head shape)",
+                      "TFLOP/s", flops / dt / 1e12, dt * 1e3, "C3-attention")
+    res["config"].update({"positions": S, "q_heads": Hq, "kv_heads": Hkv, "head_dim": D,
+                          "layout": "8 x (prompt 128 + 4 completions x 480) + padding",
+                          "visible_pairs": n_vis, "visible_fraction_of_causal": n_vis / (S * (S + 1) / 2)})
+    executed = {"attn_fwd_kernel": 2, "attn_bwd_kv_kernel": 4, "attn_bwd_dq_kernel": 3}
+    res["kernels"] = {}
+    for name, (ms, n) in prof.items():
+        launch_ms = ms / max(n, 1)
+        tf = executed[name] * unit_flops / (launch_ms * 1e-3) / 1e12
+        res["kernels"][name] = {"launch_ms": launch_ms, "tflops_executed_on_visible_pairs": tf,
+                                "frac": tf / PEAK_BF16_TFLOPS}
+    kv = res["kernels"]["attn_bwd_kv_kernel"]
+    res["roofline"] = {"kernel": "attn_bwd_kv_kernel", "bound": "mfma",
+                       "achieved": kv["tflops_executed_on_visible_pairs"], "peak": PEAK_BF16_TFLOPS,
+                       "unit": "TFLOP/s", "frac": kv["frac"], "traffic": None, "launch_ms": kv["launch_ms"]}
+    res["plan_ms"] = timed(lambda: ops.attn_plan(group.to(dev), parent.to(dev)), 3, 1) * 1e3
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import attn_oracle
+
+        # one prompt with its completions (2048 positions), all heads, dense bias, fwd + bwd
+        n = pl + nc * cl
+        sl = lambda t: t[:n].cpu()
+        t0 = time.perf_counter()
+        attn_oracle.attention_grads(sl(q), sl(k), sl(v), group[:n], parent[:n], sl(d_out))
+        cdt = time.perf_counter() - t0
+        vis_n = pl * (pl + 1) // 2 + nc * (cl * pl + cl * (cl + 1) // 2)
+        res["cpu_baseline"] = {"value": 14.0 * vis_n * D * Hq / cdt / 1e12, "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {n} positions (one prompt and its completions), all heads, "
+                                         f"dense-bias fp32 torch-CPU oracle fwd+bwd, 1 run of {cdt:.1f} s; "
+                                         "same visible-pair flop count"}
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -257,6 +338,8 @@ def main():
         return bench_lora(args)
     if args.workload == "moe":
         return bench_moe(args)
+    if args.workload == "attn":
+        return bench_attn(args)
     case = {"c1": synthetic.config1, "c3": synthetic.config3, "c4": synthetic.config4}[args.workload]()
     T, H = case.hidden.shape[1], case.hidden.shape[2]
     V = case.lm_head.shape[0]

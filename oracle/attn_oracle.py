@@ -69,3 +69,24 @@ def visible_pairs(group_ids, parent_ids) -> int:
     """Number of (query, key) pairs the bias leaves visible in one row."""
     S = group_ids.numel()
     return int(visibility(group_ids.view(1, S), parent_ids.view(1, S)).sum().item())
+
+
+def attention_rows(q, k, v, group_ids, parent_ids, rows, scale=None, dtype=torch.float32):
+    """Same as `attention` for the query positions `rows` (1-D index tensor) only:
+    out [len(rows), Hq, D], lse [Hq, len(rows)].  For sizes where the S x S bias
+    does not fit; the rule is the one of train.py:185-199 applied to the window."""
+    S, Hq, D = q.shape
+    Hkv = k.shape[1]
+    rep = Hq // Hkv
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    j = torch.arange(S).unsqueeze(0)
+    vis = (j <= rows.unsqueeze(1)) & ((group_ids[rows].unsqueeze(1) == group_ids.unsqueeze(0)) |
+                                      (parent_ids[rows].unsqueeze(1) == group_ids.unsqueeze(0)))
+    bias = torch.where(vis, torch.zeros((), dtype=dtype), torch.full((), float("-inf"), dtype=dtype))
+    qh = q[rows].to(dtype).permute(1, 0, 2)
+    kh = k.to(dtype).permute(1, 0, 2).repeat_interleave(rep, 0)
+    vh = v.to(dtype).permute(1, 0, 2).repeat_interleave(rep, 0)
+    s = qh @ kh.transpose(1, 2) * scale + bias
+    lse = torch.logsumexp(s, -1)
+    out = (torch.exp(s - lse.unsqueeze(-1)) @ vh).permute(1, 0, 2)
+    return out, lse

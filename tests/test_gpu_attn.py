@@ -120,3 +120,51 @@ def test_attn_bwd_random_ids(artk_lib, gpu):
     assert rel_l2(dq.float().cpu(), ref_dq) <= 1e-2
     assert rel_l2(dk.float().cpu(), ref_dk) <= 1e-2
     assert rel_l2(dv.float().cpu(), ref_dv) <= 1e-2
+
+
+def test_packed_attention_autograd(artk_lib, gpu):
+    """The module-level entry: batch of two packed rows, [B, H, S, D] storage, autograd."""
+    from art_amd.attention import attention_plans, packed_attention
+    B, S, Hq, Hkv, D = 2, 256, 4, 2, 64
+    g = torch.Generator().manual_seed(31)
+    mk = lambda H: torch.randn(B, H, S, D, generator=g).to(torch.bfloat16)
+    q, k, v, d_out = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    ids = [synthetic.packed_row_ids(40 + b, S, 1 + b, 20, 2, 50) for b in range(B)]
+    group = torch.stack([i[0] for i in ids])
+    parent = torch.stack([i[1] for i in ids])
+    plans = attention_plans(group.to(gpu), parent.to(gpu))
+    qd, kd, vd = (t.to(gpu).requires_grad_(True) for t in (q, k, v))
+    out = packed_attention(qd.transpose(1, 2), kd.transpose(1, 2), vd.transpose(1, 2), plans)
+    out.backward(d_out.to(gpu).transpose(1, 2))
+    for b in range(B):
+        sh = lambda t: t[b].permute(1, 0, 2)
+        ref_out, ref_dq, ref_dk, ref_dv = attn_oracle.attention_grads(sh(q), sh(k), sh(v), group[b], parent[b],
+                                                                      sh(d_out))
+        assert rel_l2(out[b].float().cpu(), ref_out) <= 1e-2
+        assert rel_l2(qd.grad[b].float().cpu().permute(1, 0, 2), ref_dq) <= 1e-2
+        assert rel_l2(kd.grad[b].float().cpu().permute(1, 0, 2), ref_dk) <= 1e-2
+        assert rel_l2(vd.grad[b].float().cpu().permute(1, 0, 2), ref_dv) <= 1e-2
+
+
+def test_attn_full_size_windows(artk_lib, gpu):
+    """Row of 16384 positions at the 7B head shape (28 query / 4 key-value heads of
+    128): windows of queries against the oracle, and properties that need no
+    oracle (padding rows see only padding; the first token of a completion
+    attends to its prompt and itself)."""
+    S, Hq, Hkv, D = 16384, 28, 4, 128
+    q, k, v = make_qkv(77, S, Hq, Hkv, D)
+    group, parent = synthetic.packed_row_ids(78, S, 8, 128, 4, 470)   # 8 * 2008 = 16064, rest padding
+    plan = ops.attn_plan(group.to(gpu), parent.to(gpu))
+    out, lse = ops.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), plan)
+    out, lse = out.float().cpu(), lse.cpu()
+    for start in (0, 2008 - 30, 128 + 470 - 8, 16064 - 40, S - 64):
+        rows = torch.arange(start, start + 64)
+        ref_out, ref_lse = attn_oracle.attention_rows(q, k, v, group, parent, rows)
+        assert (lse[:, rows] - ref_lse).abs().max().item() <= 2e-3
+        assert rel_l2(out[rows], ref_out) <= 1e-2
+    # the first padding position sees only itself: out = v of that position
+    first_pad = 16064
+    assert torch.equal(out[first_pad, :7].to(torch.bfloat16), v[first_pad, 0].expand(7, D))
+    # determinism
+    out2, _ = ops.attn_fwd(q.to(gpu), k.to(gpu), v.to(gpu), plan)
+    assert torch.equal(out2.float().cpu(), out)

@@ -86,3 +86,16 @@ def test_attention_grads_finite_difference():
             args_m = [tm if x is t else x for x in (q, k, v)]
             fd = (f(*args_p) - f(*args_m)) / (2 * eps)
             assert abs(fd.item() - grad[idx].item()) < 1e-6
+
+
+def test_attention_rows_equals_full():
+    g = torch.Generator().manual_seed(6)
+    S, Hq, Hkv, D = 64, 4, 2, 16
+    q = torch.randn(S, Hq, D, generator=g)
+    k = torch.randn(S, Hkv, D, generator=g)
+    v = torch.randn(S, Hkv, D, generator=g)
+    group, parent = synthetic.packed_row_ids(7, S, 2, 5, 2, 12)
+    out, lse = attn_oracle.attention(q, k, v, group, parent, dtype=torch.float64)
+    rows = torch.tensor([0, 4, 5, 17, 33, 58, 63])
+    o2, l2 = attn_oracle.attention_rows(q, k, v, group, parent, rows, dtype=torch.float64)
+    assert (o2 - out[rows]).abs().max().item() < 1e-12 and (l2 - lse[:, rows]).abs().max().item() < 1e-12
