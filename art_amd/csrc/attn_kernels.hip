@@ -619,6 +619,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
 }
 
 // ---- dK, dV: 128 keys x one query head per work-group, lane = key ------------
+// 8 wavefronts = 4 key groups of 32 x 2 halves of each 64-query tile, so every
+// SIMD holds two waves and the exp2 / convert work of one overlaps the MFMAs of
+// the other.  The two waves of a key group keep separate accumulators, added
+// through LDS at the end.  The K and V rows of the block stay in LDS for the
+// whole kernel (their fragments are re-read per tile: keeping them in
+// registers would push a wave past 256 registers).
 // With grouped-query heads the work-groups of the heads that share a key/value
 // head write fp32 partial sums, which attn_kv_reduce_kernel adds in a fixed order.
 // LDS stage: Q tile, dO tile (64 queries), and lse2 / delta / group / parent codes
@@ -629,74 +635,95 @@ struct AttnQStage {
   static constexpr int DO_OFF = T::BYTES;
   static constexpr int ROW_OFF = 2 * T::BYTES;
   static constexpr int STAGE = ROW_OFF + 1024;
-  static constexpr int N_PER = 2 * T::N4 + 1;
+  static constexpr int NSTAGE = 2;
+  static constexpr int KV_OFF = NSTAGE * STAGE;          // K block (2 tiles), then V block
+  static constexpr int LDS = KV_OFF + 4 * T::BYTES;
 };
 
 // DMA of one query tile into a stage: this wave's share of the Q and dO tiles and
-// one of the four per-query arrays (wave 0: lse2, 1: delta, 2: group codes, 3: parent codes).
+// one of the four per-query arrays (wave & 3 = 0: lse2, 1: delta, 2: group codes,
+// 3: parent codes; the upper four waves write the same bytes again).
 template <int D>
 __device__ __forceinline__ void attn_issue_q(char* st, int hq, int q0, __amdgpu_buffer_rsrc_t rsrc_q,
                                              __amdgpu_buffer_rsrc_t rsrc_do,
-                                             __amdgpu_buffer_rsrc_t rsrc_row,
-                                             const int* voff_q,
-                                             const int* voff_do,
-                                             const AttnBwdParams& p, int wave, int lane) {
+                                             __amdgpu_buffer_rsrc_t rsrc_row, const int* voff_q,
+                                             const int* voff_do, const AttnBwdParams& p, int wave,
+                                             int lane) {
   using T = AttnTile<D>;
   using G = AttnQStage<D>;
   const int so_q = (int)((q0 * p.q_ss + hq * p.q_hs) * 2);
   const int so_do = (int)((q0 * p.do_ss + hq * p.do_hs) * 2);
 #pragma unroll
-  for (int i = 0; i < T::N4; ++i) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, (lds_ptr_t)(st + (wave * T::N4 + i) * 1024), 16,
+  for (int i = 0; i < T::N8; ++i) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, (lds_ptr_t)(st + (wave * T::N8 + i) * 1024), 16,
                                              voff_q[i], so_q, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_do, (lds_ptr_t)(st + G::DO_OFF + (wave * T::N4 + i) * 1024),
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_do, (lds_ptr_t)(st + G::DO_OFF + (wave * T::N8 + i) * 1024),
                                              16, voff_do[i], so_do, 0, 0);
   }
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row, (lds_ptr_t)(st + G::ROW_OFF + wave * 256), 4, lane * 4,
-                                           (int)(((wave < 2 ? (int64_t)hq * p.S : 0) + q0) * 4), 0, 0);
+  const int arr = wave & 3;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row, (lds_ptr_t)(st + G::ROW_OFF + arr * 256), 4, lane * 4,
+                                           (int)(((arr < 2 ? (int64_t)hq * p.S : 0) + q0) * 4), 0, 0);
+}
+
+// The block's K and V rows (128 each = two 64-row tiles per operand).
+template <int D>
+__device__ __forceinline__ void attn_issue_kv_block(char* dst, int key0, __amdgpu_buffer_rsrc_t rsrc_k,
+                                                    __amdgpu_buffer_rsrc_t rsrc_v, const int* voff_k,
+                                                    const int* voff_v, int64_t k_ss, int64_t v_ss,
+                                                    int wave) {
+  using T = AttnTile<D>;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < T::N8; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_k, (lds_ptr_t)(dst + t * T::BYTES + (wave * T::N8 + i) * 1024), 16, voff_k[i],
+          (int)((key0 + 64 * t) * k_ss * 2), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_v, (lds_ptr_t)(dst + (2 + t) * T::BYTES + (wave * T::N8 + i) * 1024), 16, voff_v[i],
+          (int)((key0 + 64 * t) * v_ss * 2), 0, 0);
+    }
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
+__global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   using T = AttnTile<D>;
   using G = AttnQStage<D>;
-  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE];
+  __shared__ __attribute__((aligned(1024))) char smem[G::LDS];
   __shared__ uint16_t s_list[ATT_MAX_KB];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, h = lane >> 5;
+  const int kg = wave & 3, qh = wave >> 2;
   const TrLane tr(lane);
   const int hq = blockIdx.x % p.Hq;
   const int kb = (int)(blockIdx.x / p.Hq);  // early key blocks are seen by the most queries
   const int rep = p.Hq / p.Hkv;
   const int hkv = hq / rep;
-  const int key = kb * ATT_BK2 + wave * 32 + n;
+  const int key = kb * ATT_BK2 + kg * 32 + n;
   const int cnt = p.cntT[kb];
-  for (int i = threadIdx.x; i < cnt; i += 256) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
-
-  bf16x8 kf[D / 16], vf[D / 16];
-  {
-    const uint16_t* kp = p.K + (int64_t)key * p.k_ss + (int64_t)hkv * p.k_hs + 8 * h;
-    const uint16_t* vp = p.V + (int64_t)key * p.v_ss + (int64_t)hkv * p.v_hs + 8 * h;
-#pragma unroll
-    for (int s = 0; s < D / 16; ++s) {
-      kf[s] = *(const bf16x8*)(kp + 16 * s);
-      vf[s] = *(const bf16x8*)(vp + 16 * s);
-    }
-  }
+  for (int i = threadIdx.x; i < cnt; i += 512) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
   const int gk = p.gc[key];
 
   const __amdgpu_buffer_rsrc_t rsrc_q = attn_rsrc(p.Q);
   const __amdgpu_buffer_rsrc_t rsrc_do = attn_rsrc(p.dO);
-  const void* row_src = wave == 0 ? (const void*)p.lse2 : wave == 1 ? (const void*)p.delta
-                        : wave == 2 ? (const void*)p.gc : (const void*)p.pc;
+  const int arr = wave & 3;
+  const void* row_src = arr == 0 ? (const void*)p.lse2 : arr == 1 ? (const void*)p.delta
+                        : arr == 2 ? (const void*)p.gc : (const void*)p.pc;
   const __amdgpu_buffer_rsrc_t rsrc_row = attn_rsrc(row_src);
-  int voff_q[T::N4], voff_do[T::N4];
+  int voff_q[T::N8], voff_do[T::N8];
+  {
+    int voff_k[T::N8], voff_v[T::N8];
 #pragma unroll
-  for (int i = 0; i < T::N4; ++i) {
-    voff_q[i] = T::voff(wave * T::N4 + i, lane, p.q_ss);
-    voff_do[i] = T::voff(wave * T::N4 + i, lane, p.do_ss);
+    for (int i = 0; i < T::N8; ++i) {
+      voff_q[i] = T::voff(wave * T::N8 + i, lane, p.q_ss);
+      voff_do[i] = T::voff(wave * T::N8 + i, lane, p.do_ss);
+      voff_k[i] = T::voff(wave * T::N8 + i, lane, p.k_ss);
+      voff_v[i] = T::voff(wave * T::N8 + i, lane, p.v_ss);
+    }
+    attn_issue_kv_block<D>(smem + G::KV_OFF, kb * ATT_BK2, attn_rsrc(p.K + (int64_t)hkv * p.k_hs),
+                           attn_rsrc(p.V + (int64_t)hkv * p.v_hs), voff_k, voff_v, p.k_ss, p.v_ss, wave);
   }
-  __syncthreads();
+  __syncthreads();  // s_list
   auto* list_lds = s_list;
 #define ATTN_ISSUE(IT, STG)                                                                          \
   attn_issue_q<D>(smem + (STG) * G::STAGE, hq,                                                        \
@@ -709,74 +736,99 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(AttnBwdParams p) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) dk[dt][j] = dv[dt][j] = 0.f;
 
+  // this wave's keys inside the resident K / V blocks
+  const char* kblk = smem + G::KV_OFF + (kg >> 1) * T::BYTES;
+  const char* vblk = kblk + 2 * T::BYTES;
+  const int krow = 32 * (kg & 1) + n;
+
   if (cnt > 0) ATTN_ISSUE(0, 0);
-  if (cnt > 1) ATTN_ISSUE(1, 1);
-  int stage = 0;
   for (int it = 0; it < cnt; ++it) {
-    if (it + 1 < cnt)
-      wait_vmcnt<G::N_PER>();
-    else
-      wait_vmcnt<0>();
+    wait_vmcnt<0>();
     __syncthreads();
-    if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
+    if (it + 1 < cnt) ATTN_ISSUE(it + 1, (it + 1) & 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int q0 = (entry & 0x3fff) * ATT_BQ2;
     const bool partial = (entry >> 14) == 1;
-    const char* st = smem + stage * G::STAGE;
+    const char* st = smem + (it & 1) * G::STAGE;
     const char* dot = st + G::DO_OFF;
     const float* r_lse2 = (const float*)(st + G::ROW_OFF);
     const float* r_delta = r_lse2 + 64;
     const int* r_gc = (const int*)(r_lse2 + 128);
     const int* r_pc = r_gc + 64;
 
-    bf16x8 pf[4], dsf[4];
+    floatx16 sc, dp;
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      floatx16 sc, dp;
+    for (int j = 0; j < 16; ++j) sc[j] = dp[j] = 0.f;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) sc[j] = dp[j] = 0.f;
+    for (int s = 0; s < D / 16; ++s) {
+      sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::row_frag(st, 32 * qh + n, s, h),
+                                                   T::row_frag(kblk, krow, s, h), sc, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::row_frag(dot, 32 * qh + n, s, h),
+                                                   T::row_frag(vblk, krow, s, h), dp, 0, 0, 0);
+    }
+    bf16x8 pf[2], dsf[2];
 #pragma unroll
-      for (int s = 0; s < D / 16; ++s) {
-        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::row_frag(st, 32 * qt + n, s, h), kf[s], sc, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::row_frag(dot, 32 * qt + n, s, h), vf[s], dp, 0, 0, 0);
+    for (int g4 = 0; g4 < 4; ++g4) {
+      const int qi = 32 * qh + 8 * g4 + 4 * h;
+      const floatx4 l4 = *(const floatx4*)(r_lse2 + qi);
+      const floatx4 d4 = *(const floatx4*)(r_delta + qi);
+      int gq[4] = {0, 0, 0, 0}, pq[4] = {0, 0, 0, 0};
+      if (partial) {
+        const int4 a4 = *(const int4*)(r_gc + qi);
+        const int4 b4 = *(const int4*)(r_pc + qi);
+        gq[0] = a4.x; gq[1] = a4.y; gq[2] = a4.z; gq[3] = a4.w;
+        pq[0] = b4.x; pq[1] = b4.y; pq[2] = b4.z; pq[3] = b4.w;
       }
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int qi = 32 * qt + 8 * g4 + 4 * h;
-        const floatx4 l4 = *(const floatx4*)(r_lse2 + qi);
-        const floatx4 d4 = *(const floatx4*)(r_delta + qi);
-        int gq[4] = {0, 0, 0, 0}, pq[4] = {0, 0, 0, 0};
-        if (partial) {
-          const int4 a4 = *(const int4*)(r_gc + qi);
-          const int4 b4 = *(const int4*)(r_pc + qi);
-          gq[0] = a4.x; gq[1] = a4.y; gq[2] = a4.z; gq[3] = a4.w;
-          pq[0] = b4.x; pq[1] = b4.y; pq[2] = b4.z; pq[3] = b4.w;
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int j = 4 * g4 + e;
-          float x = __builtin_fmaf(sc[j], p.scale_log2e, -l4[e]);
-          if (partial && !attn_visible(q0 + qi + e, key, gq[e], pq[e], gk)) x = -INFINITY;
-          const float pr = __builtin_amdgcn_exp2f(x);
-          pf[2 * qt + j / 8][j % 8] = (__bf16)pr;
-          dsf[2 * qt + j / 8][j % 8] = (__bf16)(pr * (dp[j] - d4[e]));
-        }
+      for (int e = 0; e < 4; ++e) {
+        const int j = 4 * g4 + e;
+        float x = __builtin_fmaf(sc[j], p.scale_log2e, -l4[e]);
+        if (partial && !attn_visible(q0 + qi + e, key, gq[e], pq[e], gk)) x = -INFINITY;
+        const float pr = __builtin_amdgcn_exp2f(x);
+        pf[j / 8][j % 8] = (__bf16)pr;
+        dsf[j / 8][j % 8] = (__bf16)(pr * (dp[j] - d4[e]));
       }
     }
     // dV^T += dO^T P, dK^T += Q^T dS: transposing reads of the dO and Q tiles
 #pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2) {
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
       for (int dt = 0; dt < D / 32; ++dt) {
-        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(dot, tr, 16 * s2, 32 * dt), pf[s2], dv[dt],
-                                                         0, 0, 0);
-        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(st, tr, 16 * s2, 32 * dt), dsf[s2], dk[dt],
-                                                         0, 0, 0);
+        dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(dot, tr, 32 * qh + 16 * u, 32 * dt), pf[u],
+                                                         dv[dt], 0, 0, 0);
+        dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(st, tr, 32 * qh + 16 * u, 32 * dt), dsf[u],
+                                                         dk[dt], 0, 0, 0);
       }
     }
-    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
   }
 #undef ATTN_ISSUE
+
+  // add the accumulators of the two query halves: the upper waves park theirs in
+  // LDS ([key group][register][lane], conflict-free), the lower waves add and store
+  float* red = (float*)smem;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    __syncthreads();
+    if (qh == 1) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          red[((kg * (D / 2) + dt * 16 + j) << 6) + lane] = pass == 0 ? dk[dt][j] : dv[dt][j];
+    }
+    __syncthreads();
+    if (qh == 0) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const float v = red[((kg * (D / 2) + dt * 16 + j) << 6) + lane];
+          if (pass == 0) dk[dt][j] += v; else dv[dt][j] += v;
+        }
+    }
+  }
+  if (qh == 1) return;
+
   if (rep > 1) {
     const int64_t o = ((((int64_t)(hq - hkv * rep) * p.S + key) * p.Hkv + hkv) * D) + 4 * h;
 #pragma unroll
@@ -1042,9 +1094,9 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   p.scale_log2e = scale * LOG2E;
   prof_begin(PROF_ATTN_BWD_KV, st);
   if (D == 128)
-    attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hq), 256, 0, st>>>(p);
+    attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hq), 512, 0, st>>>(p);
   else
-    attn_bwd_kv_kernel<64><<<(unsigned)(pl.nKb2 * Hq), 256, 0, st>>>(p);
+    attn_bwd_kv_kernel<64><<<(unsigned)(pl.nKb2 * Hq), 512, 0, st>>>(p);
   prof_end(PROF_ATTN_BWD_KV, st);
   ARTK_CHECK_LAUNCH();
   if (Hq != Hkv) {
