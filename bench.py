@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe", "attn"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe", "attn", "pack"],
                     help="c3 (default, the headline): fused GRPO step at the Qwen2.5-7B shape; c1/c4: the "
                          "0.5B / 14B shapes; lora: LoRA linear fwd+bwd at the Qwen2.5-3B shapes; moe: "
                          "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
@@ -320,6 +320,59 @@ def bench_attn(args):
     print(json.dumps(res))
 
 
+def bench_pack(args):
+    """Packer (host code, no kernel): 64 prompts of 256 tokens with 8 completions of 768 tokens each,
+    packed into rows of 16384.  value = packed tokens per second of `art_amd.pack`; the baseline is the
+    list-based algorithm of the reference restated in oracle/pack_oracle.py on the same inputs."""
+    import random
+
+    import torch
+
+    from art_amd import pack
+
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import pack_oracle
+
+    g = random.Random(1007)
+    results = []
+    for pid in range(64):
+        prompt = [g.randint(0, 150000) for _ in range(256)]
+        for _ in range(8):
+            comp = [g.randint(0, 150000) for _ in range(768)]
+            results.append(pack_oracle.Result(
+                token_ids=prompt + comp, input_pos=list(range(1024)), assistant_mask=[0] * 256 + [1] * 768,
+                logprobs=[float("nan")] * 256 + [-g.random() for _ in range(768)], advantage=g.uniform(-1, 1),
+                prompt_id=pid, prompt_length=256))
+    seq_len = 16384
+    out = pack.packed_tensors_from_tokenized_results(results, seq_len, rng=random.Random(1))
+    n_tokens = int((out["group_ids"] != -1).sum())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = pack.packed_tensors_from_tokenized_results(results, seq_len, rng=random.Random(1))
+    dt = (time.perf_counter() - t0) / args.steps
+    res = base_result(args, "packer tokens/s (host)", "tokens/s", n_tokens / dt, dt * 1e3, "pack-64x8x1024")
+    res["dtype"] = "int64/f32"
+    res["config"].update({"results": len(results), "rows": out["tokens"].shape[0], "row_length": seq_len,
+                          "packed_tokens": n_tokens})
+    res["roofline"] = None  # host code: no kernel to place on a roofline
+    if torch.cuda.is_available():
+        stager = pack.RowStager(seq_len, torch.device("cuda:0"))
+        stager.to_device(out, 0)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            stager.to_device(out, 0)
+        res["row_to_device_ms"] = (time.perf_counter() - t0) / 20 * 1e3
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        ref = pack_oracle.pack(results, seq_len, rng=random.Random(1))
+        cdt = time.perf_counter() - t0
+        assert all(torch.equal(ref[k].nan_to_num(0.0) if ref[k].is_floating_point() else ref[k],
+                               out[k].nan_to_num(0.0) if out[k].is_floating_point() else out[k]) for k in ref)
+        res["cpu_baseline"] = {"value": n_tokens / cdt, "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": f"the same {len(results)} results, list-based algorithm, 1 run of {cdt:.2f} s"}
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -327,6 +380,9 @@ def main():
         print("bench.py: this build runs on ONE GPU only (the path shards over tokens with no "
               "exchange; see DESIGN.md). Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "pack":
+        return bench_pack(args)
 
     import torch
 
