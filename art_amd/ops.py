@@ -460,6 +460,35 @@ def attn_bwd(q, k, v, out, lse, d_out, plan: AttnPlan, scale: Optional[float] = 
 
 
 # -----------------------------------------------------------------------------
+# Optimizer
+# -----------------------------------------------------------------------------
+def sumsq(x: torch.Tensor) -> torch.Tensor:
+    """f32 [1]: sum of squares of a flat f32 device tensor (fixed summation order)."""
+    _need(x, "x", torch.float32)
+    lib = _lib.load()
+    out = torch.empty(1, dtype=torch.float32, device=x.device)
+    ws = _workspace(lib.artk_sumsq_f32_workspace_bytes(), x.device)
+    _lib.check(lib.artk_sumsq_f32(x.data_ptr(), x.numel(), out.data_ptr(), ws.data_ptr(), ws.numel(),
+                                  _stream(x.device)))
+    return out
+
+
+def adamw_step(p, g, m, v, p_bf16, lr, beta1, beta2, eps, weight_decay, step, grad_sumsq=None,
+               max_grad_norm=0.0) -> None:
+    """In-place fused AdamW over flat f32 buffers (see artk_adamw_step)."""
+    n = p.numel()
+    for name, t in (("p", p), ("g", g), ("m", m), ("v", v)):
+        _need(t, name, torch.float32)
+        if t.numel() != n:
+            raise ValueError(f"{name}: expected {n} elements")
+    if p_bf16 is not None:
+        _need(p_bf16, "p_bf16", torch.bfloat16)
+    _lib.check(_lib.load().artk_adamw_step(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(),
+                                           _ptr(p_bf16), n, lr, beta1, beta2, eps, weight_decay, step,
+                                           _ptr(grad_sumsq), max_grad_norm, _stream(p.device)))
+
+
+# -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------
 (PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM, PROF_ATTN_FWD,

@@ -250,6 +250,27 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
                       void* workspace, size_t workspace_bytes, artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * Optimizer step over the adapter parameters kept in one flat fp32 buffer.
+ * Replaces: the per-tensor AdamW step and gradient clipping that HF Trainer runs
+ *   with the reference's settings, src/art/dev/model.py:69-85 (betas 0.9 / 0.99,
+ *   weight_decay 0.1, max_grad_norm 0.1, constant lr; `paged_adamw_8bit` there:
+ *   the moments are kept in fp32 here).
+ * artk_sumsq_f32: out[0] = sum x[i]^2 (fixed summation order, double partials).
+ * artk_adamw_step: g' = g * min(1, max_grad_norm / (sqrt(*grad_sumsq) + 1e-6))
+ *   (no clipping when grad_sumsq is NULL); p *= 1 - lr * weight_decay;
+ *   m = m + (g' - m)(1 - beta1); v = beta2 v + (1 - beta2) g'^2;
+ *   p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps);
+ *   params_bf16 (may be NULL) receives the rounded copy of p.  step counts from 1.
+ * ------------------------------------------------------------------------- */
+size_t artk_sumsq_f32_workspace_bytes(void);
+int32_t artk_sumsq_f32(const float* x, int64_t n, float* out, void* workspace, size_t workspace_bytes,
+                       artk_stream_t stream);
+int32_t artk_adamw_step(float* params, const float* grads, float* exp_avg, float* exp_avg_sq,
+                        void* params_bf16, int64_t n, float lr, float beta1, float beta2, float eps,
+                        float weight_decay, int32_t step, const float* grad_sumsq, float max_grad_norm,
+                        artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
  * artk_profile_enable(1) makes later calls bracket each dominant kernel with
  * HIP events on the launch stream; after the caller has synchronised,
