@@ -68,6 +68,7 @@ SIGNATURES = {
     "artk_sumsq_f32_workspace_bytes": (_sz, []),
     "artk_sumsq_f32": (_i32, [_p, _i64, _p, _p, _sz, _p]),
     "artk_adamw_step": (_i32, [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _f32, _i32, _p, _f32, _p]),
+    "artk_nf4_dequant": (_i32, [_p, _p, _p, _p, _p, _f32, _i64, _i32, _p, _p]),
     "artk_transpose_bf16_batched": (_i32, [_p, _p, _i64, _i64, _i64, _p]),
     "artk_profile_enable": (_i32, [_i32]),
     "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),

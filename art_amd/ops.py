@@ -460,6 +460,28 @@ def attn_bwd(q, k, v, out, lse, d_out, plan: AttnPlan, scale: Optional[float] = 
 
 
 # -----------------------------------------------------------------------------
+# NF4 base weights
+# -----------------------------------------------------------------------------
+def nf4_dequant(packed, absmax=None, absmax_q=None, code2=None, absmax2=None, offset: float = 0.0,
+                blocksize: int = 64, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bf16 [2 * packed.numel()] from NF4 codes (see artk_nf4_dequant)."""
+    _need(packed, "packed", torch.uint8)
+    n = packed.numel() * 2
+    if absmax is not None:
+        _need(absmax, "absmax", torch.float32, (n // blocksize,))
+    else:
+        _need(absmax_q, "absmax_q", torch.uint8, (n // blocksize,))
+        _need(code2, "code2", torch.float32, (256,))
+        _need(absmax2, "absmax2", torch.float32)
+    if out is None:
+        out = torch.empty(n, dtype=torch.bfloat16, device=packed.device)
+    _lib.check(_lib.load().artk_nf4_dequant(packed.data_ptr(), _ptr(absmax), _ptr(absmax_q), _ptr(code2),
+                                            _ptr(absmax2), offset, n, blocksize, out.data_ptr(),
+                                            _stream(packed.device)))
+    return out
+
+
+# -----------------------------------------------------------------------------
 # Optimizer
 # -----------------------------------------------------------------------------
 def sumsq(x: torch.Tensor) -> torch.Tensor:

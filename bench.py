@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe", "attn", "pack", "optim"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c3", "c4", "lora", "moe", "attn", "pack", "optim", "nf4"],
                     help="c3 (default, the headline): fused GRPO step at the Qwen2.5-7B shape; c1/c4: the "
                          "0.5B / 14B shapes; lora: LoRA linear fwd+bwd at the Qwen2.5-3B shapes; moe: "
                          "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
@@ -417,6 +417,41 @@ def bench_optim(args):
     print(json.dumps(res))
 
 
+def bench_nf4(args):
+    """NF4 -> bf16 dequantisation of one gate projection of a Qwen2.5-7B (18944 x 3584, block size 64).
+    value = elements per second; roofline = HBM bytes (0.5625 B read + 2 B written per element)."""
+    import numpy as np
+    import torch
+
+    from art_amd import ops
+
+    dev = torch.device("cuda:0")
+    n = 18944 * 3584
+    g = torch.Generator().manual_seed(1009)
+    packed = torch.randint(0, 256, (n // 2,), generator=g, dtype=torch.uint8).to(dev)
+    absmax = (0.05 * torch.rand(n // 64, generator=g)).to(dev)
+    out = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    dt = timed(lambda: ops.nf4_dequant(packed, absmax, out=out), args.steps, args.warmup)
+    res = base_result(args, "NF4 dequantisation elements/s", "elements/s", n / dt, dt * 1e3, "gate-proj-7B")
+    res["dtype"] = "u8->bf16"
+    res["config"].update({"elements": n, "blocksize": 64})
+    gbs = 2.5625 * n / dt / 1e9
+    res["roofline"] = {"kernel": "nf4_dequant_kernel", "bound": "hbm", "achieved": gbs, "peak": 8000.0,
+                       "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None}
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import quant_oracle
+
+        m = 64 * 65536
+        pk, am = packed[: m // 2].cpu().numpy(), absmax[: m // 64].cpu().numpy()
+        t0 = time.perf_counter()
+        quant_oracle.to_bf16_bits(quant_oracle.dequantize(pk, am, 64))
+        cdt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": m / cdt, "unit": "elements/s", "cores": 1, "kind": "port",
+                               "sample": f"first {m} elements, numpy oracle, 1 run of {cdt:.2f} s"}
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -442,6 +477,8 @@ def main():
         return bench_attn(args)
     if args.workload == "optim":
         return bench_optim(args)
+    if args.workload == "nf4":
+        return bench_nf4(args)
     case = {"c1": synthetic.config1, "c3": synthetic.config3, "c4": synthetic.config4}[args.workload]()
     T, H = case.hidden.shape[1], case.hidden.shape[2]
     V = case.lm_head.shape[0]

@@ -271,6 +271,22 @@ int32_t artk_adamw_step(float* params, const float* grads, float* exp_avg, float
                         artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * NF4 base weight -> bf16.
+ * Replaces: the dequantisation that bitsandbytes performs in front of every
+ *   frozen linear when the base model is loaded with `load_in_4bit=True`
+ *   (src/art/dev/model.py:29); the result feeds artk_lora_linear_fwd/bwd.
+ *   packed  u8 [n/2]   two codes per byte, first element in the high nibble
+ *   absmax  f32 [n/blocksize], or NULL with the double-quantised form:
+ *   absmax_q u8 [n/blocksize], code2 f32 [256], absmax2 f32 [ceil(n/blocksize/256)],
+ *           offset:  absmax[b] = code2[absmax_q[b]] * absmax2[b / 256] + offset
+ *   out_bf16 [n] = bf16(level[code] * absmax[block])
+ * n must be a multiple of blocksize (a power of two >= 32; bitsandbytes uses 64).
+ * ------------------------------------------------------------------------- */
+int32_t artk_nf4_dequant(const void* packed, const float* absmax, const void* absmax_q,
+                         const float* code2, const float* absmax2, float offset, int64_t n,
+                         int32_t blocksize, void* out_bf16, artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
  * artk_profile_enable(1) makes later calls bracket each dominant kernel with
  * HIP events on the launch stream; after the caller has synchronised,
