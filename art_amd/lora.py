@@ -73,3 +73,70 @@ class LoRALinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return lora_linear(x, self.weight, self.lora_A, self.lora_B, self.scaling)
+
+
+class _FusedLoRAFn(torch.autograd.Function):
+    """Several projections of the same input as ONE product: the frozen weights
+    are concatenated along the output dimension, the adapters become a rank
+    sum(r_i) update whose B factor is block-diagonal."""
+
+    @staticmethod
+    def forward(ctx, x, weight_cat, scale, outs, ranks, *AB):
+        lead = x.shape[:-1]
+        n = len(outs)
+        As, Bs = AB[:n], AB[n:]
+        x2 = x.reshape(-1, x.shape[-1]).to(torch.bfloat16).contiguous()
+        A_cat = torch.cat([a.detach().to(torch.bfloat16) for a in As], 0).contiguous()
+        B_bd = torch.zeros((sum(outs), sum(ranks)), dtype=torch.bfloat16, device=x.device)
+        o0 = r0 = 0
+        for b, o, r in zip(Bs, outs, ranks):
+            B_bd[o0:o0 + o, r0:r0 + r] = b.detach().to(torch.bfloat16)
+            o0 += o
+            r0 += r
+        y, xa = ops.lora_linear_fwd(x2, weight_cat, A_cat, B_bd, scale)
+        ctx.save_for_backward(x2, weight_cat, A_cat, B_bd, xa)
+        ctx.meta = (scale, lead, outs, ranks, [a.dtype for a in As], [b.dtype for b in Bs], x.dtype)
+        return y.view(*lead, sum(outs))
+
+    @staticmethod
+    def backward(ctx, g):
+        x2, weight_cat, A_cat, B_bd, xa = ctx.saved_tensors
+        scale, lead, outs, ranks, a_dt, b_dt, x_dt = ctx.meta
+        g2 = g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous()
+        dx, dA, dB = ops.lora_linear_bwd(g2, x2, ops.transposed_weight(weight_cat), A_cat, B_bd, xa, scale)
+        dAs, dBs = [], []
+        o0 = r0 = 0
+        for o, r, ad, bd in zip(outs, ranks, a_dt, b_dt):
+            dAs.append(dA[r0:r0 + r].to(ad))
+            dBs.append(dB[o0:o0 + o, r0:r0 + r].to(bd))   # off-diagonal blocks belong to no adapter
+            o0 += o
+            r0 += r
+        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, None, None, *dAs, *dBs)
+
+
+class FusedLoRALinear(nn.Module):
+    """Projections that read the same activations (q/k/v, or gate/up) as one
+    product: one pass over x instead of one per projection, and the narrow
+    projections (k, v: 256 or 512 columns) ride in the tiles of the wide one
+    instead of leaving most of the GPU idle.  ``forward(x)`` returns the tuple of
+    the individual outputs; the parameters stay per projection."""
+
+    def __init__(self, layers):
+        super().__init__()
+        layers = list(layers)
+        if len({l.in_features for l in layers}) != 1 or len({l.scaling for l in layers}) != 1:
+            raise ValueError("fused projections need the same input size and scaling")
+        self.outs = tuple(l.out_features for l in layers)
+        self.ranks = tuple(l.r for l in layers)
+        if sum(self.ranks) > 64:
+            raise ValueError("sum of ranks above 64")
+        self.scaling = layers[0].scaling
+        self.weight = nn.Parameter(torch.cat([l.weight.detach() for l in layers], 0).contiguous(),
+                                   requires_grad=False)
+        self.lora_A = nn.ParameterList([l.lora_A for l in layers])
+        self.lora_B = nn.ParameterList([l.lora_B for l in layers])
+
+    def forward(self, x: torch.Tensor):
+        y = _FusedLoRAFn.apply(x, self.weight, float(self.scaling), self.outs, self.ranks, *self.lora_A,
+                               *self.lora_B)
+        return torch.split(y, self.outs, dim=-1)

@@ -99,3 +99,31 @@ def test_lora_module_autograd(artk_lib, gpu):
     assert rel_l2(mod.lora_A.grad.cpu(), dA0) <= TOL
     assert rel_l2(mod.lora_B.grad.cpu(), dB0) <= TOL
     assert mod.weight.grad is None
+
+
+def test_fused_projections_match_separate(artk_lib, gpu):
+    """q/k/v as one product: same outputs and gradients as three LoRALinear modules."""
+    from art_amd.lora import FusedLoRALinear, LoRALinear
+    torch.manual_seed(5)
+    T, n_in = 192, 256
+    layers = [LoRALinear(n_in, o, r=8, lora_alpha=16, device=gpu, dtype=torch.float32) for o in (256, 64, 64)]
+    for l in layers:
+        torch.nn.init.normal_(l.lora_B, std=0.05)
+    fused = FusedLoRALinear(layers)
+    x1 = torch.randn(T, n_in, device=gpu).to(torch.bfloat16).requires_grad_(True)
+    x2 = x1.detach().clone().requires_grad_(True)
+    ups = [torch.randn(T, o, device=gpu).to(torch.bfloat16) for o in (256, 64, 64)]
+    ys = [l(x1) for l in layers]
+    sum((y.float() * u.float()).sum() for y, u in zip(ys, ups)).backward()
+    ref = [(l.lora_A.grad.clone(), l.lora_B.grad.clone()) for l in layers]
+    for l in layers:
+        l.lora_A.grad = None
+        l.lora_B.grad = None
+    yf = fused(x2)
+    sum((y.float() * u.float()).sum() for y, u in zip(yf, ups)).backward()
+    rel = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
+    for a, b in zip(yf, ys):
+        assert rel(a.float(), b.float()) <= 4e-3
+    assert rel(x2.grad.float(), x1.grad.float()) <= 1e-2
+    for l, (dA, dB) in zip(layers, ref):
+        assert rel(l.lora_A.grad, dA) <= 1e-2 and rel(l.lora_B.grad, dB) <= 1e-2
