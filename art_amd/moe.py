@@ -46,6 +46,18 @@ def grouped_lora_linear(x, W, W_t, A, B, scale, routing, use_gather: bool):
     return _GroupedLoRAFn.apply(x, W, W_t, A, B, float(scale), routing, use_gather)
 
 
+def _fuse_adapters(A1, B1, A2, B2):
+    """Adapters of two projections of the same input as one of rank r1 + r2:
+    A stacked, B block-diagonal (autograd routes the gradients back to the four
+    parameters; the off-diagonal blocks of dB belong to no adapter)."""
+    A = torch.cat([A1, A2], 1)                                       # [E, r1 + r2, in]
+    E, o1, r1 = B1.shape
+    o2, r2 = B2.shape[1], B2.shape[2]
+    top = torch.cat([B1, B1.new_zeros(E, o1, r2)], 2)
+    bot = torch.cat([B2.new_zeros(E, o2, r1), B2], 2)
+    return A, torch.cat([top, bot], 1)                               # [E, o1 + o2, r1 + r2]
+
+
 class MoELoRAExperts(nn.Module):
     """E experts, each a gated MLP (gate/up [I,H], down [H,I]) with rank-r LoRA."""
 
@@ -62,6 +74,12 @@ class MoELoRAExperts(nn.Module):
             self.register_parameter(f"{name}_lora_A", nn.Parameter(
                 (torch.rand(n_experts, r, i, device=device) * 2 - 1) * bound))
             self.register_parameter(f"{name}_lora_B", nn.Parameter(torch.zeros(n_experts, o, r, device=device)))
+        # gate and up read the same rows: kept as one [E, 2I, H] weight so that they are one
+        # grouped product (one pass over x, twice the K length in the input-gradient product)
+        self.register_parameter("gate_up_weight", nn.Parameter(
+            torch.cat([self.gate_weight.detach(), self.up_weight.detach()], 1).contiguous(),
+            requires_grad=False))
+        self.intermediate = intermediate
         self._wt = {}
 
     def _transposed(self, name):
@@ -80,8 +98,10 @@ class MoELoRAExperts(nn.Module):
         """x bf16 [T,H], router_logits f32 [T,E] -> (y bf16 [T,H], routing)."""
         routing = ops.moe_route(router_logits.float().contiguous(), self.top_k)
         x = x.to(torch.bfloat16).contiguous()
-        gate = self._proj("gate", x, routing, True)
-        up = self._proj("up", x, routing, True)
+        A_gu, B_gu = _fuse_adapters(self.gate_lora_A, self.gate_lora_B, self.up_lora_A, self.up_lora_B)
+        gate_up = grouped_lora_linear(x, self.gate_up_weight, self._transposed("gate_up"), A_gu, B_gu,
+                                      self.scaling, routing, True)
+        gate, up = gate_up[:, :self.intermediate], gate_up[:, self.intermediate:]
         h = (torch.nn.functional.silu(gate.float()) * up.float()).to(torch.bfloat16)
         down = self._proj("down", h, routing, False)  # [T*k, H] in sorted order
         per_slot = down[routing.inv_perm.long()].view(x.shape[0], self.top_k, -1).float()

@@ -132,5 +132,5 @@ def test_moe_block_autograd(artk_lib, gpu):
     y0.backward(up.cpu().float())
     assert rel_l2(y.detach().cpu().float(), y0.detach()) <= 2e-2
     assert rel_l2(x.grad.cpu().float(), xr.grad) <= 2e-2
-    for n in ("gate_lora_A", "gate_lora_B", "up_lora_A", "down_lora_A", "down_lora_B"):
+    for n in ("gate_lora_A", "gate_lora_B", "up_lora_A", "up_lora_B", "down_lora_A", "down_lora_B"):
         assert rel_l2(getattr(mod, n).grad.cpu(), P[n].grad) <= 2e-2, n
