@@ -68,44 +68,71 @@ __device__ __forceinline__ bool attn_visible(int i, int j, int gi, int pi, int g
   return j <= i && (gj == gi || gj == pi);
 }
 
-// cls[qb][kb] for query blocks of BM and key blocks of BN positions:
-// 0 = no visible pair, 1 = some, 2 = all BM*BN pairs.  clsT is the transpose.
-// One wavefront per (qb, kb).
+// Visibility of one (owner block, tile) pair, per wavefront of the kernel that
+// will process it:
+//   bits 14-15  1 = some pairs visible, 2 = all
+//   bits 16-23  wave w has at least one visible pair in its part of the tile
+//   bits 24-31  every pair of wave w's part is visible (no per-element test needed)
+// 0 when nothing is visible.
+// MODE 0 (forward, dQ): owner = 256 queries, tile = 64 keys, wave w = queries 32w..32w+31.
+// MODE 1 (dK/dV):      owner = 128 keys, tile = 64 queries, wave w = keys 32(w&3).. x
+//                      queries 32(w>>2)..
+// One wavefront evaluates the rule on every pair of its (owner, tile).
+template <int MODE>
 __global__ __launch_bounds__(256) void attn_classify_kernel(const int* __restrict__ gc,
-                                                            const int* __restrict__ pc, int BM,
-                                                            int BN, int nQb, int nKb,
-                                                            uint8_t* __restrict__ cls,
-                                                            uint8_t* __restrict__ clsT) {
+                                                            const int* __restrict__ pc, int n_tile,
+                                                            uint32_t* __restrict__ info) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int kb = blockIdx.x * 4 + wave;
-  const int qb = blockIdx.y;
-  if (kb >= nKb) return;
-  int total = 0;
-  if (kb * BN <= qb * BM + BM - 1) {
-    int cnt = 0;
-    for (int kk = lane; kk < BN; kk += 64) {
-      const int j = kb * BN + kk;
+  const int tile = blockIdx.x * 4 + wave;
+  const int owner = blockIdx.y;
+  if (tile >= n_tile) return;
+  uint32_t any = 0, all = 0;
+  if (MODE == 0) {
+    const int q0 = owner * ATT_BM, j = tile * ATT_BN + lane;
+    if (tile * ATT_BN <= q0 + ATT_BM - 1) {
       const int gj = gc[j];
-      for (int ii = 0; ii < BM; ++ii) {
-        const int i = qb * BM + ii;
-        cnt += attn_visible(i, j, gc[i], pc[i], gj) ? 1 : 0;
+      for (int g = 0; g < 8; ++g) {
+        int cnt = 0;
+        for (int ii = 0; ii < 32; ++ii) {
+          const int i = q0 + 32 * g + ii;
+          cnt += attn_visible(i, j, gc[i], pc[i], gj) ? 1 : 0;
+        }
+        any |= (uint32_t)(__ballot(cnt > 0) != 0ull) << g;
+        all |= (uint32_t)(__ballot(cnt == 32) == ~0ull) << g;
       }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, 64);
-    total = cnt;
+  } else {
+    const int k0 = owner * ATT_BK2, q0 = tile * ATT_BQ2;
+    if (k0 <= q0 + ATT_BQ2 - 1) {
+      for (int iter = 0; iter < 2; ++iter) {
+        const int j = k0 + 64 * iter + lane;
+        const int gj = gc[j];
+        for (int qh = 0; qh < 2; ++qh) {
+          int cnt = 0;
+          for (int ii = 0; ii < 32; ++ii) {
+            const int i = q0 + 32 * qh + ii;
+            cnt += attn_visible(i, j, gc[i], pc[i], gj) ? 1 : 0;
+          }
+          const unsigned long long ab = __ballot(cnt > 0), fb = __ballot(cnt == 32);
+          for (int hh = 0; hh < 2; ++hh) {
+            const int bit = 2 * iter + hh + 4 * qh;
+            any |= (uint32_t)((uint32_t)(ab >> (32 * hh)) != 0u) << bit;
+            all |= (uint32_t)((uint32_t)(fb >> (32 * hh)) == 0xffffffffu) << bit;
+          }
+        }
+      }
+    }
   }
   if (lane == 0) {
-    const uint8_t c = total == 0 ? 0 : (total == BM * BN ? 2 : 1);
-    cls[(int64_t)qb * nKb + kb] = c;
-    if (clsT) clsT[(int64_t)kb * nQb + qb] = c;
+    const uint32_t cls = all == 0xffu ? 2u : 1u;
+    info[(int64_t)owner * n_tile + tile] = any ? (cls << 14) | (any << 16) | (all << 24) : 0u;
   }
 }
 
-// list[row][0..cnt[row]) = the columns of cls[row][*] that are not 0, ascending,
-// as  column | class << 14.  One work-group per row.
-__global__ __launch_bounds__(256) void attn_compact_kernel(const uint8_t* __restrict__ cls,
-                                                           int ncol, uint16_t* __restrict__ list,
+// list[row][0..cnt[row]) = tile index | info for the tiles of info[row][*] that
+// are not 0, ascending.  One work-group per row.
+__global__ __launch_bounds__(256) void attn_compact_kernel(const uint32_t* __restrict__ info, int ncol,
+                                                           uint32_t* __restrict__ list,
                                                            int* __restrict__ cnt) {
   __shared__ int wtot[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -113,7 +140,7 @@ __global__ __launch_bounds__(256) void attn_compact_kernel(const uint8_t* __rest
   int base = 0;
   for (int c0 = 0; c0 < ncol; c0 += 256) {
     const int c = c0 + threadIdx.x;
-    const int v = c < ncol ? cls[(int64_t)row * ncol + c] : 0;
+    const uint32_t v = c < ncol ? info[(int64_t)row * ncol + c] : 0u;
     const unsigned long long m = __ballot(v != 0);
     const int rank = __popcll(m & ((1ull << lane) - 1ull));
     __syncthreads();
@@ -121,7 +148,7 @@ __global__ __launch_bounds__(256) void attn_compact_kernel(const uint8_t* __rest
     __syncthreads();
     int off = base;
     for (int w = 0; w < wave; ++w) off += wtot[w];
-    if (v) list[(int64_t)row * ncol + off + rank] = (uint16_t)(c | (v << 14));
+    if (v) list[(int64_t)row * ncol + off + rank] = (uint32_t)c | v;
     base += wtot[0] + wtot[1] + wtot[2] + wtot[3];
   }
   if (threadIdx.x == 0) cnt[row] = base;
@@ -131,15 +158,14 @@ __global__ __launch_bounds__(256) void attn_compact_kernel(const uint8_t* __rest
 struct AttnPlan {
   int* gc;
   int* pc;
-  int nQb, nKb;        // forward: query blocks of 256, key blocks of 64
-  uint8_t* cls;        // [nQb][nKb]
-  uint16_t* list;      // [nQb][nKb]
+  int nQb, nKb;        // forward / dQ: query blocks of 256, key tiles of 64
+  uint32_t* info;      // [nQb][nKb]
+  uint32_t* list;      // [nQb][nKb]
   int* cnt;            // [nQb]
-  int nQb2, nKb2;      // dK/dV kernel: query tiles of 64 per key block of 128
-  uint8_t* cls2;       // [nQb2][nKb2]
-  uint8_t* cls2T;      // [nKb2][nQb2]
-  uint16_t* list2T;    // [nKb2][nQb2] query blocks per key block
-  int* cnt2T;          // [nKb2]
+  int nQb2, nKb2;      // dK/dV: key blocks of 128, query tiles of 64
+  uint32_t* info2;     // [nKb2][nQb2]
+  uint32_t* list2;     // [nKb2][nQb2]
+  int* cnt2;           // [nKb2]
 };
 
 static size_t attn_plan_layout(void* base, size_t bytes, int64_t S, AttnPlan& pl) {
@@ -150,13 +176,12 @@ static size_t attn_plan_layout(void* base, size_t bytes, int64_t S, AttnPlan& pl
   pl.nKb2 = (int)(S / ATT_BK2);
   pl.gc = ws.take<int>((size_t)S);
   pl.pc = ws.take<int>((size_t)S);
-  pl.cls = ws.take<uint8_t>((size_t)pl.nQb * pl.nKb);
-  pl.list = ws.take<uint16_t>((size_t)pl.nQb * pl.nKb);
+  pl.info = ws.take<uint32_t>((size_t)pl.nQb * pl.nKb);
+  pl.list = ws.take<uint32_t>((size_t)pl.nQb * pl.nKb);
   pl.cnt = ws.take<int>((size_t)pl.nQb);
-  pl.cls2 = ws.take<uint8_t>((size_t)pl.nQb2 * pl.nKb2);
-  pl.cls2T = ws.take<uint8_t>((size_t)pl.nQb2 * pl.nKb2);
-  pl.list2T = ws.take<uint16_t>((size_t)pl.nQb2 * pl.nKb2);
-  pl.cnt2T = ws.take<int>((size_t)pl.nKb2);
+  pl.info2 = ws.take<uint32_t>((size_t)pl.nQb2 * pl.nKb2);
+  pl.list2 = ws.take<uint32_t>((size_t)pl.nQb2 * pl.nKb2);
+  pl.cnt2 = ws.take<int>((size_t)pl.nKb2);
   return ws.ok() || base == nullptr ? ws.used : (size_t)-1;
 }
 
@@ -251,7 +276,7 @@ struct AttnFwdParams {
   int64_t q_ss, q_hs, k_ss, k_hs, v_ss, v_hs, o_ss, o_hs;
   const int* gc;
   const int* pc;
-  const uint16_t* list;
+  const uint32_t* list;
   const int* cnt;
   int S, Hq, Hkv, nQb, nKb;
   float scale_log2e;
@@ -296,8 +321,8 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
   using T = AttnTile<D>;
   using G = AttnKvStage<D>;
   __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE];
-  __shared__ uint16_t s_list[ATT_MAX_KB];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ uint32_t s_list[ATT_MAX_KB];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const TrLane tr(lane);
   const int hq = blockIdx.x % p.Hq;
@@ -351,8 +376,11 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
     if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int kb = entry & 0x3fff;
-    const bool partial = (entry >> 14) == 1;
+    const bool active = (entry >> (16 + wave)) & 1;        // this wave's 32 queries see part of the tile
+    const bool partial = !((entry >> (24 + wave)) & 1);     // ... but not all of it
     const char* st = smem + stage * G::STAGE;
+    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
+    if (!active) continue;  // nothing of this tile is visible to this wave's queries
 
     // S^T tiles: keys 0..31 and 32..63 of the block x this wave's 32 queries
     floatx16 sc[2];
@@ -422,7 +450,6 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(vt, tr, 16 * s2, 32 * dt), pf[s2], o[dt],
                                                         0, 0, 0);
     }
-    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
   }
 #undef ATTN_ISSUE
 
@@ -460,9 +487,9 @@ struct AttnBwdParams {
   int64_t q_ss, q_hs, k_ss, k_hs, v_ss, v_hs, do_ss, do_hs, dq_ss, dq_hs, dk_ss, dk_hs, dv_ss, dv_hs;
   const int* gc;
   const int* pc;
-  const uint16_t* list;    // per query block of 256: key tiles of 64
+  const uint32_t* list;    // per query block of 256: key tiles of 64
   const int* cnt;
-  const uint16_t* listT;   // per key block of 128: query tiles of 64
+  const uint32_t* listT;   // per key block of 128: query tiles of 64
   const int* cntT;
   int S, Hq, Hkv, nQb, nKb, nQb2, nKb2;
   float scale, scale_log2e;
@@ -503,8 +530,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
   using T = AttnTile<D>;
   using G = AttnKvStage<D>;
   __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE];
-  __shared__ uint16_t s_list[ATT_MAX_KB];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ uint32_t s_list[ATT_MAX_KB];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const TrLane tr(lane);
   const int hq = blockIdx.x % p.Hq;
@@ -561,9 +588,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
     if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int kb = entry & 0x3fff;
-    const bool partial = (entry >> 14) == 1;
+    const bool active = (entry >> (16 + wave)) & 1;        // this wave's 32 queries see part of the tile
+    const bool partial = !((entry >> (24 + wave)) & 1);     // ... but not all of it
     const char* st = smem + stage * G::STAGE;
     const int* codes = (const int*)(st + G::CODE_OFF);
+    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
+    if (!active) continue;
 
     bf16x8 dsf[4];
 #pragma unroll
@@ -603,7 +633,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
         dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_frag<D>(st, tr, 16 * s2, 32 * dt), dsf[s2], dq[dt],
                                                          0, 0, 0);
     }
-    stage = stage + 1 == ATT_STAGES ? 0 : stage + 1;
   }
 #undef ATTN_ISSUE
   uint16_t* op = p.dQ + (int64_t)q * p.dq_ss + (int64_t)hq * p.dq_hs + 4 * h;
@@ -690,8 +719,8 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   using T = AttnTile<D>;
   using G = AttnQStage<D>;
   __shared__ __attribute__((aligned(1024))) char smem[G::LDS];
-  __shared__ uint16_t s_list[ATT_MAX_KB];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ uint32_t s_list[ATT_MAX_KB];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int kg = wave & 3, qh = wave >> 2;
   const TrLane tr(lane);
@@ -748,13 +777,15 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
     if (it + 1 < cnt) ATTN_ISSUE(it + 1, (it + 1) & 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int q0 = (entry & 0x3fff) * ATT_BQ2;
-    const bool partial = (entry >> 14) == 1;
+    const bool active = (entry >> (16 + wave)) & 1;        // this wave's keys x query half
+    const bool partial = !((entry >> (24 + wave)) & 1);
     const char* st = smem + (it & 1) * G::STAGE;
     const char* dot = st + G::DO_OFF;
     const float* r_lse2 = (const float*)(st + G::ROW_OFF);
     const float* r_delta = r_lse2 + 64;
     const int* r_gc = (const int*)(r_lse2 + 128);
     const int* r_pc = r_gc + 64;
+    if (!active) continue;
 
     floatx16 sc, dp;
 #pragma unroll
@@ -921,15 +952,15 @@ int32_t artk_attn_plan(const int64_t* group_ids, const int64_t* parent_ids, int6
   hipStream_t st = (hipStream_t)stream;
   attn_codes_kernel<<<(unsigned)(S / 256), 256, 0, st>>>(group_ids, parent_ids, (int)S, pl.gc, pl.pc);
   ARTK_CHECK_LAUNCH();
-  attn_classify_kernel<<<dim3((unsigned)((pl.nKb + 3) / 4), (unsigned)pl.nQb), 256, 0, st>>>(
-      pl.gc, pl.pc, ATT_BM, ATT_BN, pl.nQb, pl.nKb, pl.cls, nullptr);
+  attn_classify_kernel<0><<<dim3((unsigned)((pl.nKb + 3) / 4), (unsigned)pl.nQb), 256, 0, st>>>(
+      pl.gc, pl.pc, pl.nKb, pl.info);
   ARTK_CHECK_LAUNCH();
-  attn_compact_kernel<<<(unsigned)pl.nQb, 256, 0, st>>>(pl.cls, pl.nKb, pl.list, pl.cnt);
+  attn_compact_kernel<<<(unsigned)pl.nQb, 256, 0, st>>>(pl.info, pl.nKb, pl.list, pl.cnt);
   ARTK_CHECK_LAUNCH();
-  attn_classify_kernel<<<dim3((unsigned)((pl.nKb2 + 3) / 4), (unsigned)pl.nQb2), 256, 0, st>>>(
-      pl.gc, pl.pc, ATT_BQ2, ATT_BK2, pl.nQb2, pl.nKb2, pl.cls2, pl.cls2T);
+  attn_classify_kernel<1><<<dim3((unsigned)((pl.nQb2 + 3) / 4), (unsigned)pl.nKb2), 256, 0, st>>>(
+      pl.gc, pl.pc, pl.nQb2, pl.info2);
   ARTK_CHECK_LAUNCH();
-  attn_compact_kernel<<<(unsigned)pl.nKb2, 256, 0, st>>>(pl.cls2T, pl.nQb2, pl.list2T, pl.cnt2T);
+  attn_compact_kernel<<<(unsigned)pl.nKb2, 256, 0, st>>>(pl.info2, pl.nQb2, pl.list2, pl.cnt2);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -1081,8 +1112,8 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   p.pc = pl.pc;
   p.list = pl.list;
   p.cnt = pl.cnt;
-  p.listT = pl.list2T;
-  p.cntT = pl.cnt2T;
+  p.listT = pl.list2;
+  p.cntT = pl.cnt2;
   p.S = (int)S;
   p.Hq = Hq;
   p.Hkv = Hkv;
