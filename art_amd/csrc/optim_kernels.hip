@@ -43,11 +43,11 @@ __global__ __launch_bounds__(256) void sumsq_partial_kernel(const float* __restr
 
 __global__ __launch_bounds__(64) void sumsq_final_kernel(const double* __restrict__ part,
                                                          float* __restrict__ out) {
-  if (threadIdx.x == 0) {
-    double s = 0.0;
-    for (int i = 0; i < SUMSQ_BLOCKS; ++i) s += part[i];
-    out[0] = (float)s;
-  }
+  // lane l adds its 16 consecutive partials in index order, then a fixed butterfly over the wave
+  double s = 0.0;
+  for (int i = 0; i < SUMSQ_BLOCKS / 64; ++i) s += part[threadIdx.x * (SUMSQ_BLOCKS / 64) + i];
+  s = wave_sum(s);
+  if (threadIdx.x == 0) out[0] = (float)s;
 }
 
 struct AdamWParams {
