@@ -151,20 +151,44 @@ __device__ __forceinline__ void mma_frags(TileAcc<NI>& acc, const Frags<NI>& f) 
 //                of the DMA for the stage after next goes into the freed buffer
 // The loop body has no branches: past the end, the DMA re-fetches the last
 // stage into the idle buffer and the fragment prefetch reads values nobody uses.
+// The two operand loaders and the K range of one tile.  Separate from the main
+// loop so that a kernel that walks several tiles can set up the next tile's
+// loaders (index loads and address arithmetic) while the current tile computes,
+// and start its first DMA stage before the current tile's epilogue.
 template <int NI>
-__device__ __forceinline__ void gemm_tile_nt(TileAcc<NI>& acc, char* smem, const void* P, int64_t ldp,
-                                             int64_t prow0, int64_t prows, const void* Q,
-                                             int64_t ldq, int64_t qrow0, int64_t qrows, int k_begin,
-                                             int k_end, const int* qgather = nullptr) {
+struct TileLoaders {
+  OperandLoader<NI> lp, lq;
+  int k_begin, k_end;
+  __device__ __forceinline__ void init(const void* P, int64_t ldp, int64_t prow0, int64_t prows,
+                                       const void* Q, int64_t ldq, int64_t qrow0, int64_t qrows, int kb,
+                                       int ke, const int* qgather = nullptr) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    lp.init(P, ldp, prow0, prows, wave, lane);
+    lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather);
+    k_begin = kb;
+    k_end = ke;
+  }
+  // First K stage into LDS stage 0.  No wave of the work-group may still be
+  // reading stage 0 (true at kernel start and after gemm_tile_run returns).
+  __device__ __forceinline__ void issue_first(char* smem) const {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    lp.template issue<0, 2 * NI>(smem, wave, k_begin);
+    lq.template issue<0, 2 * NI>(smem + OPER_STAGE_BYTES, wave, k_begin);
+  }
+};
+
+// Main loop over the K range of L; L.issue_first(smem) must have been called.
+template <int NI>
+__device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const TileLoaders<NI>& L) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
   constexpr int DI = 2 * NI;
-
-  OperandLoader<NI> lp, lq;
-  lp.init(P, ldp, prow0, prows, wave, lane);
-  lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather);
+  const OperandLoader<NI>& lp = L.lp;
+  const OperandLoader<NI>& lq = L.lq;
+  const int k_begin = L.k_begin, k_end = L.k_end;
 
   // Per-lane LDS read offsets (within an operand stage) for the 4 K=16 steps.
   int off[4];
@@ -181,8 +205,6 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc<NI>& acc, char* smem, const
   const int k_last = k_end - BK;
 
   constexpr int EARLY = NI;  // DMA instructions per operand issued right after the barrier
-  lp.template issue<0, DI>(smem, wave, k_begin);
-  lq.template issue<0, DI>(smem + OPER_STAGE_BYTES, wave, k_begin);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   {
@@ -269,6 +291,17 @@ __device__ __forceinline__ void gemm_tile_nt(TileAcc<NI>& acc, char* smem, const
   // Drain the redundant tail DMA before the caller reuses or releases LDS.
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
+}
+
+template <int NI>
+__device__ __forceinline__ void gemm_tile_nt(TileAcc<NI>& acc, char* smem, const void* P, int64_t ldp,
+                                             int64_t prow0, int64_t prows, const void* Q,
+                                             int64_t ldq, int64_t qrow0, int64_t qrows, int k_begin,
+                                             int k_end, const int* qgather = nullptr) {
+  TileLoaders<NI> L;
+  L.init(P, ldp, prow0, prows, Q, ldq, qrow0, qrows, k_begin, k_end, qgather);
+  L.issue_first(smem);
+  gemm_tile_run(acc, smem, L);
 }
 
 // Map the hardware's round-robin block->XCD placement (block b runs on XCD

@@ -133,27 +133,18 @@ __device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const F
   }
 }
 
+// Epilogue of one logits tile: optional bf16 stash of the rows the backward needs,
+// then the (max, sumexp) partials and the target gather.
 template <bool STASH>
-__global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
-  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  int vt, tt;
-  tile_coords(id, p.VT, p.TT, vt, tt);
-  const int n = p.rows.n();
-  if (tt * TILE >= n) return;  // compact mode: token tiles past the last row
-
-  TileAcc<FWD_NI> acc;
-  acc.zero();
-  gemm_tile_nt(acc, smem, p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0,
-               (int)p.H, p.rows.row_token);
-
+__device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt,
+                                                    int tt, int n) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave_m<FWD_NI>(wave), wn = wave_n<FWD_NI>(wave);
   const int half = lane >> 5;
   const int64_t vbase = (int64_t)vt * TILE + wm * 128;  // first vocab row of this wave
 
-  // Targets of this lane's 4 positions (issued early: consumed after the reductions).
+  // Targets of this lane's positions (issued early: consumed after the reductions).
   int64_t y[FWD_NI];
   int col[FWD_NI];
 #pragma unroll
@@ -186,11 +177,65 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
   }
 
   // The accumulators are only read from here on (writing to them would make the
-  // compiler shuttle all 256 between the accumulation and the vector registers).
+  // compiler shuttle all of them between the accumulation and the vector registers).
   if ((int64_t)vt * TILE + TILE > p.V)
     lse_epilogue<true>(acc, p, vt, wm, vbase, y, col, n);
   else
     lse_epilogue<false>(acc, p, vt, wm, vbase, y, col, n);
+}
+
+// Next tile of this work-group at or after id `t` (stride = grid size) whose
+// token tile is not past the last row; false when there is none.
+__device__ __forceinline__ bool lmhead_next_tile(const FwdParams& p, int n_tiles, int n, int& t, int& vt,
+                                                 int& tt) {
+  for (; t < n_tiles; t += gridDim.x) {
+    tile_coords(xcd_remap(t, n_tiles), p.VT, p.TT, vt, tt);
+    if (tt * TILE < n) return true;
+  }
+  return false;
+}
+
+// Persistent work-groups (one per CU): each walks tiles t, t + grid, ...  The
+// next tile's loaders are set up before the current tile's main loop and its
+// first DMA stage is started before the current tile's epilogue, so the
+// prologue latency of a tile hides behind the epilogue of the previous one.
+template <bool STASH>
+__global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int n_tiles = p.VT * p.TT;
+  const int n = p.rows.n();
+  int t = blockIdx.x, vt, tt;
+  if (!lmhead_next_tile(p, n_tiles, n, t, vt, tt)) return;
+  {
+    TileLoaders<FWD_NI> first;
+    first.init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H,
+               p.rows.row_token);
+    first.issue_first(smem);
+  }
+  for (;;) {
+    int t2 = t + gridDim.x, vt2 = 0, tt2 = 0;
+    const bool more = lmhead_next_tile(p, n_tiles, n, t2, vt2, tt2);
+    TileAcc<FWD_NI> acc;
+    acc.zero();
+    {
+      TileLoaders<FWD_NI> cur;  // its first stage is already on the way
+      cur.init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H,
+               p.rows.row_token);
+      gemm_tile_run(acc, smem, cur);
+    }
+    if (more) {
+      // loaders are rebuilt rather than kept: alive through the epilogue they cost registers
+      TileLoaders<FWD_NI> nxt;
+      nxt.init(p.W, p.H, (int64_t)vt2 * TILE, p.V, p.hidden, p.H, (int64_t)tt2 * TILE, n, 0, (int)p.H,
+               p.rows.row_token);
+      nxt.issue_first(smem);
+    }
+    lmhead_fwd_epilogue<STASH>(acc, p, vt, tt, n);
+    if (!more) break;
+    t = t2;
+    vt = vt2;
+    tt = tt2;
+  }
 }
 
 // K2: merge the per-tile (max, sumexp) partials of each position.  A block
@@ -771,7 +816,8 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   p.TT = (int)((Tc + TILE - 1) / TILE);
   fill_f32_kernel<<<(unsigned)((Tc + 255) / 256), 256, 0, st>>>(sel, Tc, NAN);
   ARTK_CHECK_LAUNCH();
-  const unsigned grid = (unsigned)(p.VT * p.TT);
+  const int n_tiles = p.VT * p.TT;
+  const unsigned grid = (unsigned)(n_tiles < num_cus() ? n_tiles : num_cus());
   prof_begin(PROF_LMHEAD_FWD, st);
   if (stash)
     lmhead_fwd_kernel<true><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
