@@ -34,21 +34,13 @@ struct LoraGemmParams {
   int r, RP, MT, NT;
 };
 
-__global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemmParams p) {
-  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  int mt, nt;
-  tile_coords(id, p.MT, p.NT, mt, nt);
+// Rank-r steps and bf16 store of one finished tile.
+__device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const LoraGemmParams& p, int mt,
+                                                   int nt) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave_m<LORA_NI>(wave), wn = wave_n<LORA_NI>(wave);
   const int half = lane >> 5;
-
-  TileAcc<LORA_NI> acc;
-  acc.zero();
-  gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
-               (int)p.K);
-
   if (p.Pe != nullptr) {
     int64_t prow[4], qrow[LORA_NI];
 #pragma unroll
@@ -79,6 +71,44 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemm
         for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
         *(bf16x4*)(p.out + col * p.M + m) = o;
       }
+  }
+}
+
+// Persistent work-groups: tiles t, t + grid, ...; the first DMA stage of the next
+// tile is started before the rank-r steps and the store of the current one.
+__global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemmParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int n_tiles = p.MT * p.NT;
+  int t = blockIdx.x;
+  int mt, nt;
+  tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt);
+  {
+    TileLoaders<LORA_NI> first;
+    first.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
+    first.issue_first(smem);
+  }
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const bool more = t2 < n_tiles;
+    int mt2 = 0, nt2 = 0;
+    if (more) tile_coords(xcd_remap(t2, n_tiles), p.MT, p.NT, mt2, nt2);
+    TileAcc<LORA_NI> acc;
+    acc.zero();
+    {
+      TileLoaders<LORA_NI> cur;  // its first stage is already on the way
+      cur.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
+      gemm_tile_run(acc, smem, cur);
+    }
+    if (more) {
+      TileLoaders<LORA_NI> nxt;
+      nxt.init(p.P, p.K, (int64_t)mt2 * TILE, p.M, p.Q, p.K, (int64_t)nt2 * TILE, p.N, 0, (int)p.K);
+      nxt.issue_first(smem);
+    }
+    lora_gemm_epilogue(acc, p, mt, nt);
+    if (!more) break;
+    t = t2;
+    mt = mt2;
+    nt = nt2;
   }
 }
 
@@ -237,7 +267,14 @@ static int32_t launch_lora_gemm(const void* P, const void* Q, const uint16_t* Pe
   p.MT = (int)((M + TILE - 1) / TILE);
   p.NT = (int)((N + TILE - 1) / TILE);
   prof_begin(PROF_LORA_GEMM, st);
-  lora_gemm_kernel<<<(unsigned)(p.MT * p.NT), nthreads<LORA_NI>(), 0, st>>>(p);
+  {
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    const int n_tiles = p.MT * p.NT;
+    lora_gemm_kernel<<<(unsigned)(n_tiles < cus ? n_tiles : cus), nthreads<LORA_NI>(), 0, st>>>(p);
+  }
   prof_end(PROF_LORA_GEMM, st);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;

@@ -177,57 +177,103 @@ struct MoeGemmParams {
   int E, r, RP, MT;
 };
 
+// One tile of the grouped product: expert, rows and weight tile.
+struct MoeTile {
+  int e, mt, nvalid;
+  int64_t row0, row_end;
+};
+
+__device__ __forceinline__ MoeTile moe_tile(const MoeGemmParams& p, int t, int n_work) {
+  const int id = xcd_remap(t, n_work);
+  const int rt = id / p.MT;
+  MoeTile m;
+  m.mt = id - rt * p.MT;
+  m.e = find_group(p.tile_prefix, p.E, rt);
+  m.row0 = p.offsets[m.e] + (int64_t)(rt - p.tile_prefix[m.e]) * TILE;
+  m.row_end = p.offsets[m.e + 1];
+  m.nvalid = (int)(m.row_end - m.row0 < TILE ? m.row_end - m.row0 : TILE);
+  return m;
+}
+
+__device__ __forceinline__ void moe_tile_loaders(TileLoaders<MOE_NI>& L, const MoeGemmParams& p,
+                                                 const MoeTile& m) {
+  L.init((const char*)p.W + (int64_t)m.e * p.M * p.K * 2, p.K, (int64_t)m.mt * TILE, p.M, p.X, p.K, m.row0,
+         m.row_end, 0, (int)p.K, p.gather);
+}
+
+// Persistent work-groups: tiles t, t + grid, ... of the device-side work list; the
+// next tile's first DMA stage starts before the rank-r steps and the store of the
+// current one (short K loops: 12 or 32 steps per tile).
 __global__ __launch_bounds__(nthreads<MOE_NI>()) void moe_gemm_kernel(MoeGemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int n_work = p.tile_prefix[p.E] * p.MT;
-  if ((int)blockIdx.x >= n_work) return;
-  const int id = xcd_remap(blockIdx.x, n_work);
-  const int rt = id / p.MT, mt = id - rt * p.MT;
-  const int e = find_group(p.tile_prefix, p.E, rt);
-  const int64_t row0 = p.offsets[e] + (int64_t)(rt - p.tile_prefix[e]) * TILE;
-  const int64_t row_end = p.offsets[e + 1];
-  const int nvalid = (int)(row_end - row0 < TILE ? row_end - row0 : TILE);
-
+  int t = blockIdx.x;
+  if (t >= n_work) return;
+  MoeTile cur = moe_tile(p, t, n_work);
+  {
+    TileLoaders<MOE_NI> first;
+    moe_tile_loaders(first, p, cur);
+    first.issue_first(smem);
+  }
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave_m<MOE_NI>(wave), wn = wave_n<MOE_NI>(wave);
   const int half = lane >> 5;
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const bool more = t2 < n_work;
+    MoeTile nxt = cur;
+    if (more) nxt = moe_tile(p, t2, n_work);
 
-  TileAcc<MOE_NI> acc;
-  acc.zero();
-  gemm_tile_nt(acc, smem, (const char*)p.W + (int64_t)e * p.M * p.K * 2, p.K, (int64_t)mt * TILE, p.M,
-               p.X, p.K, row0, row_end, 0, (int)p.K, p.gather);
-
-  if (p.Pe != nullptr) {
-    int64_t prow[4], qrow[MOE_NI];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
-      prow[i] = r < p.M ? r : p.M - 1;
+    TileAcc<MOE_NI> acc;
+    acc.zero();
+    {
+      TileLoaders<MOE_NI> L;  // its first stage is already on the way
+      moe_tile_loaders(L, p, cur);
+      gemm_tile_run(acc, smem, L);
     }
-#pragma unroll
-    for (int i = 0; i < MOE_NI; ++i) {
-      int c = acc_col<MOE_NI>(wn, i, lane);
-      qrow[i] = row0 + (c < nvalid ? c : nvalid - 1);
+    if (more) {
+      TileLoaders<MOE_NI> L;
+      moe_tile_loaders(L, p, nxt);
+      L.issue_first(smem);
     }
-    lowrank_steps(acc, p.Pe + (int64_t)e * p.M * p.r, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
-  }
 
+    const int e = cur.e, mt = cur.mt, nvalid = cur.nvalid;
+    const int64_t row0 = cur.row0;
+    if (p.Pe != nullptr) {
+      int64_t prow[4], qrow[MOE_NI];
 #pragma unroll
-  for (int ni = 0; ni < MOE_NI; ++ni) {
-    const int c = acc_col<MOE_NI>(wn, ni, lane);
-    if (c >= nvalid) continue;
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
-        if (m >= p.M) continue;
-        bf16x4 o;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = (__bf16)acc.c[mi][ni][q * 4 + k];
-        *(bf16x4*)(p.out + (row0 + c) * p.M + m) = o;
+      for (int i = 0; i < 4; ++i) {
+        int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
+        prow[i] = r < p.M ? r : p.M - 1;
       }
+#pragma unroll
+      for (int i = 0; i < MOE_NI; ++i) {
+        int c = acc_col<MOE_NI>(wn, i, lane);
+        qrow[i] = row0 + (c < nvalid ? c : nvalid - 1);
+      }
+      lowrank_steps(acc, p.Pe + (int64_t)e * p.M * p.r, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
+    }
+
+#pragma unroll
+    for (int ni = 0; ni < MOE_NI; ++ni) {
+      const int c = acc_col<MOE_NI>(wn, ni, lane);
+      if (c >= nvalid) continue;
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
+          if (m >= p.M) continue;
+          bf16x4 o;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o[k] = (__bf16)acc.c[mi][ni][q * 4 + k];
+          *(bf16x4*)(p.out + (row0 + c) * p.M + m) = o;
+        }
+    }
+    if (!more) break;
+    t = t2;
+    cur = nxt;
   }
 }
 
@@ -395,7 +441,15 @@ static int32_t launch_moe_gemm(const void* W, const void* X, const int* gather, 
   p.MT = (int)((M + TILE - 1) / TILE);
   const int64_t max_row_tiles = (n_rows + TILE - 1) / TILE + E;
   prof_begin(PROF_MOE_GEMM, st);
-  moe_gemm_kernel<<<(unsigned)(max_row_tiles * p.MT), nthreads<MOE_NI>(), 0, st>>>(p);
+  {
+    // persistent: one work-group per CU walks the device-side work list
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    const int64_t upper = (int64_t)max_row_tiles * p.MT;
+    moe_gemm_kernel<<<(unsigned)(upper < cus ? upper : cus), nthreads<MOE_NI>(), 0, st>>>(p);
+  }
   prof_end(PROF_MOE_GEMM, st);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
