@@ -314,23 +314,25 @@ __global__ __launch_bounds__(256) void moe_rowdot16_kernel(
 // Grouped column products over the rows of one expert:
 //   out_e[c, r] = scale * sum_{i in rows(e)} X[row(i), c] Y[i, r]    r in [r0, r0+8)
 // out is [E,C,R], or [E,R,C] when transpose_out.  A block owns 128 columns of one
-// expert: 64 column pairs x 4 row groups (row group g takes rows g, g+4, ...),
-// merged through LDS in a fixed order.
+// expert: 16 column groups of 8 (one 16-byte load per row) x 16 row groups (row
+// group g takes rows g, g+16, ...), merged in a fixed order: butterflies over the
+// 4 row groups of a wave, then the 4 waves through LDS.
 __global__ __launch_bounds__(256) void moe_coldot8_kernel(
     const uint16_t* __restrict__ X, const int* __restrict__ gather, const float* __restrict__ Y,
     const int* __restrict__ offsets, int64_t C, int R, float scale, int transpose_out,
     float* __restrict__ out) {
   __shared__ float ys[128][8];
   __shared__ int rows[128];
-  __shared__ float red[3][64][17];
-  const int cp = threadIdx.x & 63, rg = threadIdx.x >> 6;
-  const int64_t c = ((int64_t)blockIdx.x * 64 + cp) * 2;
+  __shared__ float red[3][16][65];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cg = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const int64_t c = ((int64_t)blockIdx.x * 16 + cg) * 8;
   const int e = blockIdx.y;
   const int r0 = blockIdx.z * 8;
   const int64_t begin = offsets[e], end = offsets[e + 1];
-  float acc[2][8];
+  float acc[8][8];  // [column][r]
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < 8; ++j)
 #pragma unroll
     for (int q = 0; q < 8; ++q) acc[j][q] = 0.f;
   for (int64_t s0 = begin; s0 < end; s0 += 128) {
@@ -347,36 +349,51 @@ __global__ __launch_bounds__(256) void moe_coldot8_kernel(
     __syncthreads();
     if (c < C) {
 #pragma unroll 4
-      for (int rr = rg; rr < nrows; rr += 4) {
-        float x0, x1;
-        unpack2(*(const uint32_t*)(X + (int64_t)rows[rr] * C + c), x0, x1);
+      for (int rr = rg; rr < nrows; rr += 16) {
+        const uint4 xv = *(const uint4*)(X + (int64_t)rows[rr] * C + c);
+        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
         const floatx4 ya = *(const floatx4*)&ys[rr][0];
         const floatx4 yb = *(const floatx4*)&ys[rr][4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          acc[0][q] += x0 * ya[q];
-          acc[1][q] += x1 * ya[q];
-          acc[0][4 + q] += x0 * yb[q];
-          acc[1][4 + q] += x1 * yb[q];
+        for (int j = 0; j < 4; ++j) {
+          float x0, x1;
+          unpack2(xw[j], x0, x1);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            acc[2 * j][q] += x0 * ya[q];
+            acc[2 * j + 1][q] += x1 * ya[q];
+            acc[2 * j][4 + q] += x0 * yb[q];
+            acc[2 * j + 1][4 + q] += x1 * yb[q];
+          }
         }
       }
     }
   }
-  if (rg > 0) {
+  // the 4 row groups of a wave sit 16 lanes apart
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < 8; ++j)
 #pragma unroll
-      for (int q = 0; q < 8; ++q) red[rg - 1][cp][j * 8 + q] = acc[j][q];
+    for (int q = 0; q < 8; ++q) {
+      float v = acc[j][q];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      acc[j][q] = v;
+    }
+  if (wave > 0 && lane < 16) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int q = 0; q < 8; ++q) red[wave - 1][cg][j * 8 + q] = acc[j][q];
   }
   __syncthreads();
-  if (rg != 0 || c >= C) return;
+  if (wave != 0 || lane >= 16 || c >= C) return;
   float* oe = out + (int64_t)e * C * R;
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < 8; ++j)
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const float v =
-          (acc[j][q] + red[0][cp][j * 8 + q] + red[1][cp][j * 8 + q] + red[2][cp][j * 8 + q]) * scale;
+          (acc[j][q] + red[0][cg][j * 8 + q] + red[1][cg][j * 8 + q] + red[2][cg][j * 8 + q]) * scale;
       if (transpose_out)
         oe[(int64_t)(r0 + q) * C + c + j] = v;
       else
