@@ -41,6 +41,8 @@ def parse():
                          "expert-LoRA grouped GEMMs at the Qwen3-30B-A3B-style share")
     ap.add_argument("--chunk-tokens", type=int, default=0, help="positions per logits scratch chunk")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the secondary figures (c3/c1/c4: the skip_inactive variant), e.g. when profiling")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run one plain device copy of this size (scales FETCH_SIZE/WRITE_SIZE "
@@ -550,16 +552,18 @@ def main():
 
     # Secondary figure (never `value`): the same batch with the projection restricted to the
     # positions that can contribute to the loss; same loss and gradient, less work.
-    for _ in range(args.warmup):
-        step(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(True)
-    torch.cuda.synchronize()
-    dt_skip = time.perf_counter() - t0
-    step()  # leave the dense results in `out`
-    torch.cuda.synchronize()
+    dt_skip = None
+    if not args.no_secondary:
+        for _ in range(args.warmup):
+            step(True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(True)
+        torch.cuda.synchronize()
+        dt_skip = time.perf_counter() - t0
+        step()  # leave the dense results in `out`
+        torch.cuda.synchronize()
 
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T / (dt / args.steps)
@@ -614,9 +618,10 @@ def main():
         },
     }
     assert t_active == t_active_dense
-    result["skip_inactive"] = {"value": T / (dt_skip / args.steps), "unit": "tokens/s",
-                               "ms_per_step": dt_skip / args.steps * 1e3,
-                               "note": "flag ARTK_FUSED_SKIP_INACTIVE; batch tokens per second"}
+    if dt_skip is not None:
+        result["skip_inactive"] = {"value": T / (dt_skip / args.steps), "unit": "tokens/s",
+                                   "ms_per_step": dt_skip / args.steps * 1e3,
+                                   "note": "flag ARTK_FUSED_SKIP_INACTIVE; batch tokens per second"}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens)
     print(json.dumps(result))
