@@ -137,24 +137,10 @@ __device__ __forceinline__ void mma_frags(TileAcc<NI>& acc, const Frags<NI>& f) 
       acc.c[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.p[mi], f.q[ni], acc.c[mi][ni], 0, 0, 0);
 }
 
-// Main loop: acc += P[prow0 : prow0+256, k_begin : k_end] * Q[qrow0 : qrow0+256, same]^T.
-// k_begin/k_end are multiples of BK, k_end > k_begin.  `smem` is GEMM_LDS_BYTES
-// of LDS, 1 KiB aligned.
-//
-// Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 8 MFMAs each per wave):
-//   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read;
-//                the second half of the DMA for the next stage is issued here
-//   wait for own LDS reads and own DMA, barrier:
-//                every wave holds its step-3 fragments in registers, so the
-//                current stage is free, and the next stage has landed
-//   step 3     : MFMAs while step 0 of the next stage is read; the first half
-//                of the DMA for the stage after next goes into the freed buffer
-// The loop body has no branches: past the end, the DMA re-fetches the last
-// stage into the idle buffer and the fragment prefetch reads values nobody uses.
 // The two operand loaders and the K range of one tile.  Separate from the main
 // loop so that a kernel that walks several tiles can set up the next tile's
-// loaders (index loads and address arithmetic) while the current tile computes,
-// and start its first DMA stage before the current tile's epilogue.
+// loaders and start its first DMA stage before the current tile's epilogue
+// (its prologue latency then hides behind that epilogue).
 template <int NI>
 struct TileLoaders {
   OperandLoader<NI> lp, lq;
@@ -178,7 +164,21 @@ struct TileLoaders {
   }
 };
 
-// Main loop over the K range of L; L.issue_first(smem) must have been called.
+// Main loop over the K range of L (L.issue_first(smem) must have been called by
+// every wave): acc += P[prow0 : prow0+256, k_begin : k_end] * Q[qrow0 : qrow0+256, same]^T.
+// k_begin/k_end are multiples of BK, k_end > k_begin.  `smem` is GEMM_LDS_BYTES
+// of LDS, 1 KiB aligned.
+//
+// Schedule of one K-step (BK = 64 = 4 MFMA steps of K = 16, 8 MFMAs each per wave):
+//   steps 0..2 : MFMAs of step kk while the fragments of step kk+1 are read;
+//                the second half of the DMA for the next stage is issued here
+//   wait for own LDS reads and own DMA, barrier:
+//                every wave holds its step-3 fragments in registers, so the
+//                current stage is free, and the next stage has landed
+//   step 3     : MFMAs while step 0 of the next stage is read; the first half
+//                of the DMA for the stage after next goes into the freed buffer
+// The loop body has no branches: past the end, the DMA re-fetches the last
+// stage into the idle buffer and the fragment prefetch reads values nobody uses.
 template <int NI>
 __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const TileLoaders<NI>& L) {
   const int tid = threadIdx.x;
