@@ -18,6 +18,8 @@
 // running rescale of O^T is a per-lane scalar.  K tiles ([key][d]) and V^T
 // tiles ([d][key], from a transposed copy of V made once per call) are brought
 // into a 3-stage LDS ring by buffer_load ... lds.
+#include <stdlib.h>
+
 #include "common.hpp"
 #include "gemm_nt.hpp"
 
@@ -28,7 +30,11 @@ constexpr int ATT_BN = 64;     // keys per tile
 constexpr int ATT_STAGES = 3;
 constexpr int ATT_MAX_KB = 1024;  // key blocks per row the list in LDS can hold
 constexpr int ATT_BQ2 = 64;    // dK/dV kernel: queries per tile
-constexpr int ATT_BK2 = 128;   // dK/dV kernel: keys per work-group (4 waves x 32)
+constexpr int ATT_BK2 = 128;   // dK/dV kernel: keys per work-group (4 key groups x 32)
+// dK/dV with grouped-query heads: a key block seen by at most this many (query
+// tile, head) pairs is handled by ONE work-group for all heads of its group (no
+// partial sums); busier blocks get one work-group per head.
+constexpr int ATT_LIGHT_MAX = 64;
 
 // ----------------------------------------------------------------------------
 // Plan
@@ -492,6 +498,7 @@ struct AttnBwdParams {
   const uint32_t* listT;   // per key block of 128: query tiles of 64
   const int* cntT;
   int S, Hq, Hkv, nQb, nKb, nQb2, nKb2;
+  int light_max;           // see ATT_LIGHT_MAX; 0 when there are too few key blocks to fill the GPU that way
   float scale, scale_log2e;
 };
 
@@ -730,6 +737,9 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   const int hkv = hq / rep;
   const int key = kb * ATT_BK2 + kg * 32 + n;
   const int cnt = p.cntT[kb];
+  const bool light = rep > 1 && cnt * rep <= p.light_max;
+  if (light && hq != hkv * rep) return;  // the group's first head does all of them
+  const int nheads = light ? rep : 1;
   for (int i = threadIdx.x; i < cnt; i += 512) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
   const int gk = p.gc[key];
 
@@ -754,10 +764,14 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   }
   __syncthreads();  // s_list
   auto* list_lds = s_list;
+  // step IT of the flattened (head, visible query tile) sequence
 #define ATTN_ISSUE(IT, STG)                                                                          \
-  attn_issue_q<D>(smem + (STG) * G::STAGE, hq,                                                        \
-                  __builtin_amdgcn_readfirstlane(list_lds[IT] & 0x3fff) * ATT_BQ2, rsrc_q, rsrc_do,   \
-                  rsrc_row, voff_q, voff_do, p, wave, lane)
+  do {                                                                                               \
+    const int hi_ = (IT) / cnt, ti_ = (IT) - hi_ * cnt;                                               \
+    attn_issue_q<D>(smem + (STG) * G::STAGE, hq + hi_,                                                \
+                    __builtin_amdgcn_readfirstlane(list_lds[ti_] & 0x3fff) * ATT_BQ2, rsrc_q, rsrc_do, \
+                    rsrc_row, voff_q, voff_do, p, wave, lane);                                        \
+  } while (0)
 
   floatx16 dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -770,12 +784,15 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   const char* vblk = kblk + 2 * T::BYTES;
   const int krow = 32 * (kg & 1) + n;
 
-  if (cnt > 0) ATTN_ISSUE(0, 0);
-  for (int it = 0; it < cnt; ++it) {
+  const int total = cnt * nheads;
+  if (total > 0) ATTN_ISSUE(0, 0);
+  int ti = 0;
+  for (int it = 0; it < total; ++it) {
     wait_vmcnt<0>();
     __syncthreads();
-    if (it + 1 < cnt) ATTN_ISSUE(it + 1, (it + 1) & 1);
-    const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
+    if (it + 1 < total) ATTN_ISSUE(it + 1, (it + 1) & 1);
+    const int entry = __builtin_amdgcn_readfirstlane(s_list[ti]);
+    ti = ti + 1 == cnt ? 0 : ti + 1;
     const int q0 = (entry & 0x3fff) * ATT_BQ2;
     const bool active = (entry >> (16 + wave)) & 1;        // this wave's keys x query half
     const bool partial = !((entry >> (24 + wave)) & 1);
@@ -860,7 +877,7 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   }
   if (qh == 1) return;
 
-  if (rep > 1) {
+  if (rep > 1 && !light) {
     const int64_t o = ((((int64_t)(hq - hkv * rep) * p.S + key) * p.Hkv + hkv) * D) + 4 * h;
 #pragma unroll
     for (int dt = 0; dt < D / 32; ++dt)
@@ -897,7 +914,9 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
 // dK = scale * sum_r pK[r], dV = sum_r pV[r] over the query heads r of a group, in
 // index order; 4 elements per thread.
 __global__ __launch_bounds__(256) void attn_kv_reduce_kernel(const float* __restrict__ pK,
-                                                             const float* __restrict__ pV, int rep,
+                                                             const float* __restrict__ pV,
+                                                             const int* __restrict__ cntT,
+                                                             int light_max, int rep,
                                                              int64_t S, int Hkv, int D, float scale,
                                                              uint16_t* __restrict__ dK, int64_t dk_ss,
                                                              int64_t dk_hs, uint16_t* __restrict__ dV,
@@ -909,6 +928,7 @@ __global__ __launch_bounds__(256) void attn_kv_reduce_kernel(const float* __rest
   const int c = (int)(i % d4);
   const int hh = (int)((i / d4) % Hkv);
   const int64_t s = i / ((int64_t)d4 * Hkv);
+  if (cntT[s / ATT_BK2] * rep <= light_max) return;  // written directly by the dK/dV kernel
   floatx4 a = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
   for (int r = 0; r < rep; ++r) {
     a += ((const floatx4*)pK)[(int64_t)r * n + i];
@@ -1123,6 +1143,15 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   p.nKb2 = pl.nKb2;
   p.scale = scale;
   p.scale_log2e = scale * LOG2E;
+  {
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    p.light_max = pl.nKb2 * Hkv >= cus ? ATT_LIGHT_MAX : 0;
+    // tuning / test knob: ARTK_ATTN_LIGHT_MAX=<n> forces the threshold
+    if (const char* e = getenv("ARTK_ATTN_LIGHT_MAX")) p.light_max = atoi(e);
+  }
   prof_begin(PROF_ATTN_BWD_KV, st);
   if (D == 128)
     attn_bwd_kv_kernel<128><<<(unsigned)(pl.nKb2 * Hq), 512, 0, st>>>(p);
@@ -1133,7 +1162,7 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
   if (Hq != Hkv) {
     const int64_t n4 = S * Hkv * (D / 4);
     attn_kv_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(
-        pk, pv, Hq / Hkv, S, Hkv, D, scale, (uint16_t*)dk, strides[12], strides[13], (uint16_t*)dv,
+        pk, pv, pl.cnt2, p.light_max, Hq / Hkv, S, Hkv, D, scale, (uint16_t*)dk, strides[12], strides[13], (uint16_t*)dv,
         strides[14], strides[15]);
     ARTK_CHECK_LAUNCH();
   }
