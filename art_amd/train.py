@@ -263,10 +263,13 @@ def get_compute_loss_fn(trainer) -> Callable[..., torch.Tensor]:
             inputs["advantages"], inputs["assistant_mask"], inputs["weights"], epsilon, epsilon_high,
             ref_logprobs, config.beta, skip_inactive=True)  # new_logprobs are not used here
 
+        # The reference appends `.item()` values here (train.py:147-150), one device
+        # synchronisation per metric and step; the device scalars are kept instead and
+        # converted when `log` averages them.
         trainer._metrics["learning_rate"].append(config.learning_rate)
-        trainer._metrics["policy_loss"].append(metrics["policy_loss"].item())
+        trainer._metrics["policy_loss"].append(metrics["policy_loss"].detach())
         if config.beta > 0.0:
-            trainer._metrics["kl_div"].append(metrics["kl_div"].item())
+            trainer._metrics["kl_div"].append(metrics["kl_div"].detach())
         return loss
 
     return compute_loss
@@ -277,7 +280,7 @@ def get_log_fn(trainer, results_queue) -> Callable[..., None]:
     (reference: src/art/local/train.py:156-174)."""
 
     def log(logs, start_time=None) -> None:
-        metrics = {key: sum(vals) / len(vals) for key, vals in trainer._metrics.items()}
+        metrics = {key: float(sum(vals) / len(vals)) for key, vals in trainer._metrics.items()}
         if next(iter(logs.keys())).startswith("eval_"):
             metrics = {f"eval_{key}": val for key, val in metrics.items()}
         merged = {**logs, **metrics}
