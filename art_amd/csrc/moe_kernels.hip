@@ -130,20 +130,32 @@ __global__ __launch_bounds__(256) void moe_scan_kernel(const int* __restrict__ c
   }
 }
 
+// Stable placement of one chunk: position = base[chunk][key] + number of earlier
+// entries of the chunk with the same key.  That rank is the count in the earlier
+// waves (per-wave histograms in LDS) plus the count among the earlier lanes of the
+// own wave (64 shuffles), instead of a scan over the whole chunk per thread.
 __global__ __launch_bounds__(PERM_CHUNK) void moe_scatter_kernel(const int* __restrict__ keys, int n,
                                                                  int E, int k,
                                                                  const int* __restrict__ base,
                                                                  int* __restrict__ perm,
                                                                  int* __restrict__ inv_perm,
                                                                  int* __restrict__ row_token) {
-  __shared__ int ks[PERM_CHUNK];
+  constexpr int NW = PERM_CHUNK / 64;
+  __shared__ int hist[NW][256];  // E <= 256
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < NW * 256; i += PERM_CHUNK) (&hist[0][0])[i] = 0;
+  __syncthreads();
   const int f = blockIdx.x * PERM_CHUNK + threadIdx.x;
   const int key = f < n ? keys[f] : -1;
-  ks[threadIdx.x] = key;
-  __syncthreads();
+  if (key >= 0) atomicAdd(&hist[wave][key], 1);
   int rank = 0;
-  for (int j = 0; j < PERM_CHUNK; ++j) rank += (j < (int)threadIdx.x && ks[j] == key) ? 1 : 0;
+  for (int j = 0; j < 64; ++j) {
+    const int kj = __shfl(key, j, 64);
+    rank += (j < lane && kj == key) ? 1 : 0;
+  }
+  __syncthreads();
   if (f < n) {
+    for (int w = 0; w < wave; ++w) rank += hist[w][key];
     const int pos = base[blockIdx.x * E + key] + rank;
     perm[pos] = f;
     inv_perm[f] = pos;
