@@ -100,7 +100,7 @@ def make_grpo_case(name: str, seed: int, T: int, H: int, V: int, n_traj: int, gr
         traj_advantages=adv, noise=noise)
 
 
-# The benchmark configurations (sizes from the task's BASELINE.json).
+# The benchmark configurations.
 def config1() -> GRPOCase:
     """Qwen2.5-0.5B shape: 4 trajectories of 512 tokens, one group of 4, ~50 % mask."""
     return make_grpo_case("C1-qwen2.5-0.5b", 1001, 2048, 896, 151936, 4, 4, 0.5)

@@ -474,12 +474,68 @@ def bench_nf4(args):
     print(json.dumps(res))
 
 
+class GpuStateSampler:
+    """Polls the amdgpu hwmon files (shader clock, socket power, power cap) from a thread
+    while a burst of steps runs; sysfs reads only, no GPU runtime calls.  Fields that the
+    box does not expose are left out."""
+
+    def __init__(self, period_s=0.01):
+        import glob
+        self.period = period_s
+        self.files = {}
+        for hw in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            for key, names in (("sclk_mhz", ("freq1_input",)), ("power_w", ("power1_average", "power1_input")),
+                               ("power_cap_w", ("power1_cap",))):
+                for n in names:
+                    p = os.path.join(hw, n)
+                    if key not in self.files and os.path.exists(p):
+                        self.files[key] = p
+            if self.files:
+                break
+        self.samples = {k: [] for k in self.files}
+        self._stop = False
+        self._thread = None
+
+    def _read(self):
+        for k, p in self.files.items():
+            try:
+                with open(p) as f:
+                    self.samples[k].append(float(f.read().strip()) / 1e6)  # Hz -> MHz, uW -> W
+            except (OSError, ValueError):
+                pass
+
+    def _run(self):
+        while not self._stop:
+            self._read()
+            time.sleep(self.period)
+
+    def __enter__(self):
+        import threading
+        if self.files:
+            self._thread = threading.Thread(target=self._run, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread is not None:
+            self._thread.join()
+
+    def summary(self):
+        out = {}
+        for k, v in self.samples.items():
+            if v:
+                v = sorted(v)
+                out[k] = {"median": v[len(v) // 2], "min": v[0], "max": v[-1], "samples": len(v)}
+        return out or None
+
+
 def main():
     args = parse()
     world = int(os.environ.get("WORLD_SIZE", "1"))
     if args.gpus != 1 or world != 1:
         print("bench.py: this build runs on ONE GPU only (the path shards over tokens with no "
-              "exchange; see DESIGN.md). Re-run with --gpus 1.", file=sys.stderr)
+              "exchange, which is not built). Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     if args.workload == "pack":
@@ -539,16 +595,30 @@ def main():
         step()
     torch.cuda.synchronize()
     ops.profile_enable(True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
     fwd_ms, fwd_n = ops.profile_collect(ops.PROF_LMHEAD_FWD)
     bwd_ms, bwd_n = ops.profile_collect(ops.PROF_DHIDDEN_GEMM)
     sm_ms, sm_n = ops.profile_collect(ops.PROF_SOFTMAX_GRAD)
     ops.profile_enable(False)
-    t_active_dense = int(out[0][3].item())
+    mask_count = int(out[0][3].item())
+    # positions whose loss coefficient is non-zero (masked in, non-zero advantage, unclipped):
+    # exactly the rows with a non-zero d_hidden row, which are the rows the backward GEMM runs
+    t_active_dense = int((out[2] != 0).any(dim=1).sum().item())
+
+    # Clock and power while the same step runs back to back (its own burst, outside the timing).
+    with GpuStateSampler() as sampler:
+        for _ in range(max(args.steps, 10)):
+            step()
+        torch.cuda.synchronize()
+    gpu_state = sampler.summary()
 
     # Secondary figure (never `value`): the same batch with the projection restricted to the
     # positions that can contribute to the loss; same loss and gradient, less work.
@@ -569,7 +639,7 @@ def main():
     tokens_per_s = T / (dt / args.steps)
     # rows whose loss coefficient is zero (non-assistant positions) have a zero d_hidden row
     # and are skipped by the backward: the algorithmic work counts them in the forward only
-    t_active = int(out[0][3].item())
+    t_active = int((out[2] != 0).any(dim=1).sum().item())
     alg_flops_step = 2.0 * T * V * H + 2.0 * t_active * V * H
     # dominant kernel: one launch covers `chunk` positions against the whole vocabulary
     fwd_launch_ms = fwd_ms / max(fwd_n, 1)
@@ -589,6 +659,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_median": step_ms[len(step_ms) // 2],
+        "ms_per_step_min": step_ms[0],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -596,7 +668,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": case.name, "tokens": T, "hidden": H, "vocab": V,
                    "chunk_tokens": chunk, "mask_fraction": float(case.assistant_mask.float().mean()),
-                   "t_active": t_active},
+                   "mask_count": mask_count, "t_active": t_active},
         "algorithmic_flops_per_step": alg_flops_step,
         "tflops_algorithmic": alg_flops_step / (dt / args.steps) / 1e12,
         "frac_of_bf16_peak": alg_flops_step / (dt / args.steps) / 1e12 / PEAK_BF16_TFLOPS,
@@ -618,6 +690,8 @@ def main():
         },
     }
     assert t_active == t_active_dense
+    if gpu_state:
+        result["gpu_state_under_load"] = gpu_state
     if dt_skip is not None:
         result["skip_inactive"] = {"value": T / (dt_skip / args.steps), "unit": "tokens/s",
                                    "ms_per_step": dt_skip / args.steps * 1e3,

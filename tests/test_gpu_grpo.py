@@ -238,7 +238,7 @@ def test_fused_skip_inactive(artk_lib, gpu, T, H, V, n_traj, chunk_tokens, densi
 
 
 def test_config1_full_size(artk_lib, gpu):
-    """BASELINE config 1 (Qwen2.5-0.5B shape) at full size against the oracle."""
+    """Benchmark config 1 (Qwen2.5-0.5B shape) at full size against the oracle."""
     print("config1 full size", flush=True)
     case = synthetic.config1()
     ref = oracle_case(case, 1024)
@@ -253,7 +253,7 @@ def test_config1_full_size(artk_lib, gpu):
 
 
 # ---------------------------------------------------------------------------------
-# Full-size configurations (BASELINE configs 3 and 4): the CPU oracle cannot run the
+# Full-size configurations (benchmark configs 3 and 4): the CPU oracle cannot run the
 # whole case in seconds, so parity is checked on windows of positions (every
 # position's logprob and d_hidden row depend on the rest of the batch only through
 # the scalar mask count) and through size-independent properties.

@@ -70,7 +70,7 @@ def test_lora_zero_factors(artk_lib, gpu):
 
 @pytest.mark.parametrize("n_out", [2048, 256, 11008])
 def test_lora_config2_full_size(artk_lib, gpu, n_out):
-    """BASELINE config 2 (Qwen2.5-3B projections) at full size."""
+    """Benchmark config 2 (Qwen2.5-3B projections) at full size."""
     print(f"lora config2 out={n_out}", flush=True)
     x, W, A, B, up = make(8192, 2048, n_out, 8, 1002 + n_out)
     y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, 2.0, up)

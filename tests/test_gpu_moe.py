@@ -84,7 +84,7 @@ def test_grouped_lora_matches_oracle(artk_lib, gpu, T, H, I, E, k, use_gather):
 
 
 def test_config5_gate_projection_full_size(artk_lib, gpu):
-    """BASELINE config 5: 8192 tokens, hidden 2048, 128 experts, top-8, gate [768,2048]."""
+    """Benchmark config 5: 8192 tokens, hidden 2048, 128 experts, top-8, gate [768,2048]."""
     print("moe config5 gate projection", flush=True)
     T, H, I, E, k = 8192, 2048, 768, 128, 8
     g = torch.Generator().manual_seed(1005)
