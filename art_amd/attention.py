@@ -12,7 +12,11 @@ from typing import List, Optional
 
 import torch
 
+import torch.nn.functional as F
+
 from . import ops
+
+ROW_MULTIPLE = 256  # the kernels take rows whose length is a multiple of this
 
 
 def attention_plans(group_ids: torch.Tensor, parent_ids: torch.Tensor) -> List[ops.AttnPlan]:
@@ -21,6 +25,16 @@ def attention_plans(group_ids: torch.Tensor, parent_ids: torch.Tensor) -> List[o
     batch; every layer and head reuses them."""
     if group_ids.dim() == 1:
         group_ids, parent_ids = group_ids.unsqueeze(0), parent_ids.unsqueeze(0)
+    S = group_ids.shape[1]
+    extra = -S % ROW_MULTIPLE
+    if extra:
+        # Rows of any length: append positions whose ids no real position carries (as group
+        # or as parent), so they see and are seen by nothing but themselves; packed_attention
+        # pads q, k, v to match and drops their outputs.
+        fill = (torch.minimum(group_ids.amin(), parent_ids.amin()) - 1).reshape(1, 1)
+        fill = fill.expand(group_ids.shape[0], extra)
+        group_ids = torch.cat([group_ids, fill], 1)
+        parent_ids = torch.cat([parent_ids, fill], 1)
     return [ops.attn_plan(g.contiguous(), p.contiguous()) for g, p in zip(group_ids, parent_ids)]
 
 
@@ -49,6 +63,20 @@ def packed_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plans: L
     a [B, H, S, D] tensor goes in as ``t.transpose(1, 2)``).  Returns [B, S, Hq, D] bf16.
     Differentiable w.r.t. q, k, v."""
     if q.dim() == 3:
-        return _PackedAttentionFn.apply(q, k, v, plans[0], scale)
-    outs = [_PackedAttentionFn.apply(q[b], k[b], v[b], plans[b], scale) for b in range(q.shape[0])]
+        return _row(q, k, v, plans[0], scale)
+    outs = [_row(q[b], k[b], v[b], plans[b], scale) for b in range(q.shape[0])]
     return torch.stack(outs, 0)
+
+
+def _row(q, k, v, plan, scale):
+    S = q.shape[0]
+    extra = plan.S - S
+    if extra == 0:
+        return _PackedAttentionFn.apply(q, k, v, plan, scale)
+    if not 0 < extra < ROW_MULTIPLE:
+        raise ValueError(f"plan made for a row of {plan.S} positions, tensors have {S}")
+    if scale is None:
+        scale = float(q.shape[-1]) ** -0.5
+    pad = (0, 0, 0, 0, 0, extra)  # zero rows at the end of the sequence dimension
+    out = _PackedAttentionFn.apply(F.pad(q, pad), F.pad(k, pad), F.pad(v, pad), plan, scale)
+    return out[:S]

@@ -146,6 +146,32 @@ def test_packed_attention_autograd(artk_lib, gpu):
         assert rel_l2(vd.grad[b].float().cpu().permute(1, 0, 2), ref_dv) <= 1e-2
 
 
+@pytest.mark.parametrize("S", [200, 300, 1000])
+def test_packed_attention_any_row_length(artk_lib, gpu, S):
+    """Row lengths that are not a multiple of the kernels' 256: the wrapper appends positions
+    nothing real can see; out and gradients of the real positions match the oracle on the
+    unpadded row (padding ids of the packer, -1, included at the end of the real row)."""
+    from art_amd.attention import attention_plans, packed_attention
+    print(f"packed_attention S={S}", flush=True)
+    Hq, Hkv, D = 4, 2, 64
+    g = torch.Generator().manual_seed(77 + S)
+    mk = lambda H: torch.randn(S, H, D, generator=g).to(torch.bfloat16)
+    q, k, v, d_out = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    group, parent = synthetic.packed_row_ids(50 + S, S, 2, S // 10, 2, S // 6)
+    assert (group == -1).any()  # the packer's own padding is part of the case
+    plans = attention_plans(group.to(gpu), parent.to(gpu))
+    assert plans[0].S % 256 == 0 and plans[0].S - S < 256
+    qd, kd, vd = (t.to(gpu).requires_grad_(True) for t in (q, k, v))
+    out = packed_attention(qd, kd, vd, plans)
+    assert out.shape == (S, Hq, D)
+    out.backward(d_out.to(gpu))
+    ref_out, ref_dq, ref_dk, ref_dv = attn_oracle.attention_grads(q, k, v, group, parent, d_out)
+    assert rel_l2(out.float().cpu(), ref_out) <= 1e-2
+    assert rel_l2(qd.grad.float().cpu(), ref_dq) <= 1e-2
+    assert rel_l2(kd.grad.float().cpu(), ref_dk) <= 1e-2
+    assert rel_l2(vd.grad.float().cpu(), ref_dv) <= 1e-2
+
+
 def test_attn_full_size_windows(artk_lib, gpu):
     """Row of 16384 positions at the 7B head shape (28 query / 4 key-value heads of
     128): windows of queries against the oracle, and properties that need no
