@@ -88,7 +88,8 @@ def test_logprob_invalid_id_is_nan(artk_lib, gpu):
 
 
 @pytest.mark.parametrize("T,H,V,n_traj,chunk_tokens", [(512, 256, 8192, 4, 4096), (768, 192, 8000, 4, 256),
-                                                       (1024, 128, 4096, 8, 384)])
+                                                       (1024, 128, 4096, 8, 384), (1000, 192, 8000, 4, 0),
+                                                       (520, 64, 4160, 4, 200)])
 def test_fused_matches_oracle(artk_lib, gpu, T, H, V, n_traj, chunk_tokens):
     print(f"fused T={T} H={H} V={V} chunk={chunk_tokens}", flush=True)
     case = synthetic.make_grpo_case("t", T + H, T, H, V, n_traj, 4, 0.5)
