@@ -474,6 +474,36 @@ def bench_nf4(args):
     print(json.dumps(res))
 
 
+def torch_same_algorithm_step(hidden, lm_head, tokens, old, adv, mask, weights, chunk=1024, eps=0.2):
+    """The reference's own algorithm for this path, written with stock torch ops and run on the
+    same GPU (src/art/local/train.py:111-151, 245-285): per chunk of positions a bf16 matmul
+    against the transposed lm_head view, gather, logsumexp; then the clipped loss on the shifted
+    tensors and autograd back to the hidden states.  The reference itself cannot be imported
+    (its dependencies are absent), so this is a baseline of the method, not of its code."""
+    import torch
+    import torch.nn.functional as F
+
+    shifted = lambda t, pad: F.pad(t[:, 1:], (0, 1), value=pad)
+    hs = hidden.detach().unsqueeze(0).requires_grad_(True)             # [1, T, H]
+    head_t = lm_head.t()                                               # [H, V] view of [V, H]
+    ids = shifted(tokens.unsqueeze(0), 0)
+    parts = []
+    for h_c, id_c in zip(hs.split(chunk, 1), ids.split(chunk, 1)):
+        logits = h_c @ head_t
+        parts.append(logits.gather(-1, id_c.unsqueeze(-1)).squeeze(-1) - logits.logsumexp(-1))
+    new = torch.cat(parts, 1)
+    old_s = shifted(old.unsqueeze(0), 0.0)
+    adv_s = shifted(adv.unsqueeze(0), 0.0)
+    m = shifted(mask.unsqueeze(0), False).to(new.dtype)
+    w = shifted(weights.unsqueeze(0), 0.0)
+    old_s = torch.where(torch.isnan(old_s), new.detach(), old_s)
+    ratio = torch.exp(new - old_s)
+    pl = -torch.minimum(ratio * adv_s, ratio.clip(1 - eps, 1 + eps) * adv_s) * w * m
+    loss = pl.sum() / (m.sum() + 1e-6)
+    loss.backward()
+    return loss.detach(), hs.grad
+
+
 class GpuStateSampler:
     """Polls the amdgpu hwmon files (shader clock, socket power, power cap) from a thread
     while a burst of steps runs; sysfs reads only, no GPU runtime calls.  Fields that the
@@ -635,6 +665,23 @@ def main():
         step()  # leave the dense results in `out`
         torch.cuda.synchronize()
 
+    # Secondary figure: the reference's method in stock torch ops on this GPU.
+    torch_ms = None
+    if not args.no_secondary:
+        targs = (hidden, lm_head, tokens, old, adv, mask, weights)
+        t_loss, t_grad = torch_same_algorithm_step(*targs)   # warm-up, also a cross-check
+        torch.cuda.synchronize()
+        t_rel = ((t_grad[0].float() - out[2].float()).norm() / out[2].float().norm()).item()
+        n_rep = 3
+        t0 = time.perf_counter()
+        for _ in range(n_rep):
+            torch_same_algorithm_step(*targs)
+        torch.cuda.synchronize()
+        torch_ms = (time.perf_counter() - t0) / n_rep * 1e3
+        torch_note = (f"bf16 matmul/gather/logsumexp per 1024 positions + autograd; d_hidden rel-L2 "
+                      f"against the kernels {t_rel:.1e}; loss {float(t_loss):.6f}")
+        del t_grad
+
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = T / (dt / args.steps)
     # rows whose loss coefficient is zero (non-assistant positions) have a zero d_hidden row
@@ -696,6 +743,9 @@ def main():
         result["skip_inactive"] = {"value": T / (dt_skip / args.steps), "unit": "tokens/s",
                                    "ms_per_step": dt_skip / args.steps * 1e3,
                                    "note": "flag ARTK_FUSED_SKIP_INACTIVE; batch tokens per second"}
+    if torch_ms is not None:
+        result["torch_gpu_same_algorithm"] = {"value": T / (torch_ms * 1e-3), "unit": "tokens/s",
+                                              "ms_per_step": torch_ms, "note": torch_note}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens)
     print(json.dumps(result))
