@@ -137,6 +137,32 @@ __device__ __forceinline__ void mma_frags(TileAcc<NI>& acc, const Frags<NI>& f) 
       acc.c[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.p[mi], f.q[ni], acc.c[mi][ni], 0, 0, 0);
 }
 
+// bf16 store of one 32x32 accumulator block whose 32 rows are contiguous in the
+// output (dst = this lane's column, block row 0; 16-byte aligned).  Lanes l and
+// l + 32 hold the same column, each 4 rows of every 8.  They trade halves
+// (v_permlane32_swap), so that every lane stores 8 consecutive rows as 16 bytes:
+// rows 16p .. 16p+7 from the lower lane, 16p+8 .. 16p+15 from the upper one, and a
+// store instruction puts down 32 contiguous bytes per column instead of 16.
+// Both lanes of a pair must call it together.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+  return *(uint32_t*)&v;
+}
+__device__ __forceinline__ void store_block_bf16(uint16_t* dst, const floatx16& c, int half) {
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const uint32_t a0 = pack_bf16x2(c[8 * p + 0], c[8 * p + 1]), a1 = pack_bf16x2(c[8 * p + 2], c[8 * p + 3]);
+    const uint32_t b0 = pack_bf16x2(c[8 * p + 4], c[8 * p + 5]), b1 = pack_bf16x2(c[8 * p + 6], c[8 * p + 7]);
+    // swap(a, b): a' = {lower lanes: own a, upper lanes: the lower lane's b},
+    //             b' = {lower lanes: the upper lane's a, upper lanes: own b}
+    const auto r0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+    const auto r1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+    const uint4 v = {r0[0], r1[0], r0[1], r1[1]};
+    *(uint4*)(dst + 16 * p + 8 * half) = v;
+  }
+}
+
 // The two operand loaders and the K range of one tile.  Separate from the main
 // loop so that a kernel that walks several tiles can set up the next tile's
 // loaders and start its first DMA stage before the current tile's epilogue

@@ -20,12 +20,20 @@ __device__ __forceinline__ void lowrank_steps(TileAcc<NI>& acc, const uint16_t* 
   const int half = (threadIdx.x & 63) >> 5;
   for (int e0 = 0; e0 < rp; e0 += 16) {
     const int e = e0 + half * 8;
+    // Every lane loads (a chunk past the end reads chunk 0 instead and is zeroed
+    // afterwards): loads under a lane mask would each be waited for in turn.
+    const bool p_ok = e < pe_valid, q_ok = e < qe_valid;
+    const int ep = p_ok ? e : 0, eq = q_ok ? e : 0;
     Frags<NI> f;
     const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) f.p[i] = e < pe_valid ? *(const bf16x8*)(Pe + prow[i] * pe_ld + e) : z;
+    for (int i = 0; i < 4; ++i) f.p[i] = *(const bf16x8*)(Pe + prow[i] * pe_ld + ep);
 #pragma unroll
-    for (int i = 0; i < NI; ++i) f.q[i] = e < qe_valid ? *(const bf16x8*)(Qe + qrow[i] * qe_ld + e) : z;
+    for (int i = 0; i < NI; ++i) f.q[i] = *(const bf16x8*)(Qe + qrow[i] * qe_ld + eq);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.p[i] = p_ok ? f.p[i] : z;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) f.q[i] = q_ok ? f.q[i] : z;
     mma_frags(acc, f);
   }
 }

@@ -58,19 +58,28 @@ __device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const 
 
 #pragma unroll
   for (int ni = 0; ni < LORA_NI; ++ni) {
+    // lanes l and l + 32 share the column, so they take these branches together
+    // (store_block_bf16 exchanges data between them)
     const int64_t col = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, ni, lane);
-    if (col >= p.N) continue;
+    const bool col_ok = col < p.N;
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+    for (int mi = 0; mi < 4; ++mi) {
+      const int64_t m0 = (int64_t)mt * TILE + wm * 128 + mi * 32;
+      if (m0 >= p.M) continue;  // wave-uniform
+      if (m0 + 32 <= p.M) {
+        if (col_ok) store_block_bf16(p.out + col * p.M + m0, acc.c[mi][ni], half);
+      } else {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
-        if (m >= p.M) continue;
-        bf16x4 o;
+        for (int q = 0; q < 4; ++q) {
+          const int64_t m = m0 + q * 8 + half * 4;
+          if (m >= p.M || !col_ok) continue;
+          bf16x4 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
-        *(bf16x4*)(p.out + col * p.M + m) = o;
+          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
+          *(bf16x4*)(p.out + col * p.M + m) = o;
+        }
       }
+    }
   }
 }
 

@@ -269,19 +269,28 @@ __global__ __launch_bounds__(nthreads<MOE_NI>()) void moe_gemm_kernel(MoeGemmPar
 
 #pragma unroll
     for (int ni = 0; ni < MOE_NI; ++ni) {
+      // lanes l and l + 32 share the column, so they take these branches together
+      // (store_block_bf16 exchanges data between them)
       const int c = acc_col<MOE_NI>(wn, ni, lane);
-      if (c >= nvalid) continue;
+      const bool col_ok = c < nvalid;
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
+      for (int mi = 0; mi < 4; ++mi) {
+        const int64_t m0 = (int64_t)mt * TILE + wm * 128 + mi * 32;
+        if (m0 >= p.M) continue;  // wave-uniform
+        if (m0 + 32 <= p.M) {
+          if (col_ok) store_block_bf16(p.out + (row0 + c) * p.M + m0, acc.c[mi][ni], half);
+        } else {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 32 + q * 8 + half * 4;
-          if (m >= p.M) continue;
-          bf16x4 o;
+          for (int q = 0; q < 4; ++q) {
+            const int64_t m = m0 + q * 8 + half * 4;
+            if (m >= p.M || !col_ok) continue;
+            bf16x4 o;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) o[k] = (__bf16)acc.c[mi][ni][q * 4 + k];
-          *(bf16x4*)(p.out + (row0 + c) * p.M + m) = o;
+            for (int k = 0; k < 4; ++k) o[k] = (__bf16)acc.c[mi][ni][q * 4 + k];
+            *(bf16x4*)(p.out + (row0 + c) * p.M + m) = o;
+          }
         }
+      }
     }
     if (!more) break;
     t = t2;
