@@ -157,6 +157,22 @@ def bench_lora(args):
     res["roofline"] = {"kernel": "lora_gemm_kernel (gate/up, fwd and dx launches)", "bound": "mfma",
                        "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                        "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms}
+    if not args.no_secondary:
+        # The LoRA linear the way peft evaluates it, in stock torch ops on the same GPU:
+        # base(x) + scale * lora_B(lora_A(x)), autograd for dx, dA, dB (W frozen).
+        import torch.nn.functional as F
+
+        def torch_step():
+            for _, _, W, _, A, B, up in shapes:
+                xg = x.detach().requires_grad_(True)
+                Ag, Bg = A.detach().requires_grad_(True), B.detach().requires_grad_(True)
+                y = F.linear(xg, W) + scale * F.linear(F.linear(xg, Ag), Bg)
+                y.backward(up)
+
+        tdt = timed(torch_step, max(args.steps // 2, 3), 2)
+        res["torch_gpu_same_algorithm"] = {"value": total / tdt / 1e12, "unit": "TFLOP/s", "ms_per_step": tdt * 1e3,
+                                           "note": "F.linear(x, W) + s * F.linear(F.linear(x, A), B) with autograd "
+                                                   "(dx, dA, dB), bf16, same six projections"}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import lora_oracle
@@ -289,6 +305,7 @@ def bench_attn(args):
 
     def step():
         out, lse = ops.attn_fwd(q, k, v, plan)
+        state["fwd"] = (out, lse)
         state["grads"] = ops.attn_bwd(q, k, v, out, lse, d_out, plan)
 
     for _ in range(args.warmup):
@@ -323,6 +340,37 @@ def bench_attn(args):
                        "achieved": kv["tflops_executed_on_visible_pairs"], "peak": PEAK_BF16_TFLOPS,
                        "unit": "TFLOP/s", "frac": kv["frac"], "traffic": None, "launch_ms": kv["launch_ms"]}
     res["plan_ms"] = timed(lambda: ops.attn_plan(group.to(dev), parent.to(dev)), 3, 1) * 1e3
+    if not args.no_secondary:
+        # The reference's method on the same GPU: the dense [1, S, S] bias of calculate_attn_bias
+        # (src/art/local/train.py:177-215) handed to torch's scaled_dot_product_attention.
+        import torch.nn.functional as F
+
+        from art_amd.train import calculate_attn_bias
+
+        def torch_step(bias):
+            qh, kh, vh = (t.detach().transpose(0, 1).unsqueeze(0).requires_grad_(True) for t in (q, k, v))
+            o = F.scaled_dot_product_attention(qh, kh, vh, attn_mask=bias.unsqueeze(1), enable_gqa=True)
+            o.backward(d_out.transpose(0, 1).unsqueeze(0))
+            return o
+
+        try:
+            t0 = time.perf_counter()
+            bias = calculate_attn_bias(1, S, dev, group.view(1, S).to(dev), parent.view(1, S).to(dev),
+                                       torch.bfloat16)
+            torch.cuda.synchronize()
+            bias_ms = (time.perf_counter() - t0) * 1e3
+            o_ref = torch_step(bias)
+            rel = ((o_ref[0].transpose(0, 1).float() - state["fwd"][0].float()).norm()
+                   / state["fwd"][0].float().norm()).item()
+            tdt = timed(lambda: torch_step(bias), 3, 0)
+            res["torch_gpu_same_algorithm"] = {
+                "value": flops / tdt / 1e12, "unit": "TFLOP/s", "ms_per_step": tdt * 1e3,
+                "bias_ms": bias_ms, "bias_bytes": bias.numel() * bias.element_size(),
+                "note": f"dense bf16 bias + torch SDPA (enable_gqa) fwd+bwd, same visible-pair flop count; "
+                        f"out rel-L2 against the kernels {rel:.1e}"}
+            del bias, o_ref
+        except Exception as e:  # the baseline is informative only
+            res["torch_gpu_same_algorithm"] = {"error": f"{type(e).__name__}: {e}"[:200]}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import attn_oracle
