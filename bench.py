@@ -261,6 +261,38 @@ def bench_moe(args):
     res["roofline"] = {"kernel": "moe_gemm_kernel (mean of the 6 launches per step)", "bound": "mfma",
                        "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                        "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms}
+    if not args.no_secondary:
+        # The same work the way a stock torch MoE layer does it: softmax -> top-k, stable sort by
+        # expert, then a Python loop over the experts with F.linear on each expert's rows, autograd
+        # for dx, dA_e, dB_e (weights frozen).
+        import torch.nn.functional as F
+
+        def torch_step():
+            probs = torch.softmax(logits, -1)
+            topv, topi = torch.topk(probs, k, -1)
+            order = torch.sort(topi.reshape(-1), stable=True).indices
+            row_token = order // k
+            counts = torch.bincount(topi.reshape(-1), minlength=E).tolist()
+            xs = x[row_token].detach().requires_grad_(True)
+            hs = h.detach().requires_grad_(True)
+            params = [t.detach().requires_grad_(True) for t in (Ag, Bg, Au, Bu, Ad, Bd)]
+            a_g, b_g, a_u, b_u, a_d, b_d = params
+            outs, grads, lo = [], [], 0
+            for e in range(E):
+                hi = lo + counts[e]
+                xe, he = xs[lo:hi], hs[lo:hi]
+                yg = F.linear(xe, Wg[e]) + scale * F.linear(F.linear(xe, a_g[e]), b_g[e])
+                yu = F.linear(xe, Wu[e]) + scale * F.linear(F.linear(xe, a_u[e]), b_u[e])
+                yd = F.linear(he, Wd[e]) + scale * F.linear(F.linear(he, a_d[e]), b_d[e])
+                outs += [yg, yu, yd]
+                grads += [g_i[lo:hi], g_i[lo:hi], g_h[lo:hi]]
+                lo = hi
+            torch.autograd.backward(outs, grads)
+
+        tdt = timed(torch_step, 3, 1)
+        res["torch_gpu_same_algorithm"] = {"value": flops / tdt / 1e12, "unit": "TFLOP/s", "ms_per_step": tdt * 1e3,
+                                           "note": "softmax/top-k/stable sort + per-expert F.linear loop with "
+                                                   "autograd, bf16, same three projections"}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import moe_oracle
