@@ -16,7 +16,7 @@ namespace artk {
 // Work-group shape of each GEMM kernel (see gemm_nt.hpp).
 constexpr int FWD_NI = 2;   // lm_head projection + log-sum-exp epilogue: 8 waves
 constexpr int BWD_NI = 2;   // d_hidden GEMM
-constexpr int GEMM_NI = 4;  // plain GEMM
+constexpr int GEMM_NI = 2;  // plain GEMM
 
 // ----------------------------------------------------------------------------
 // index helpers

@@ -19,7 +19,7 @@
 
 namespace artk {
 
-constexpr int LORA_NI = 4;  // work-group shape of the LoRA GEMMs (see gemm_nt.hpp)
+constexpr int LORA_NI = 2;  // 8 waves, 2 per SIMD (see gemm_nt.hpp)
 
 // ----------------------------------------------------------------------------
 // out[n, m] = sum_k Q[n,k] P[m,k] + sum_e Qe[n,e] Pe[m,e]     (bf16 out)

@@ -21,7 +21,7 @@ namespace artk {
 // ----------------------------------------------------------------------------
 // Routing: one wavefront per token.
 // ----------------------------------------------------------------------------
-constexpr int MOE_NI = 4;  // work-group shape of the grouped GEMMs (see gemm_nt.hpp)
+constexpr int MOE_NI = 2;  // 8 waves, 2 per SIMD (see gemm_nt.hpp)
 constexpr int MOE_MAX_E = 256;
 constexpr int MOE_MAX_K = 16;
 
