@@ -196,6 +196,39 @@ def test_attn_full_size_windows(artk_lib, gpu):
     assert torch.equal(out2.float().cpu(), out)
 
 
+def test_attn_longest_row_windows_and_sums(artk_lib, gpu):
+    """The longest row the kernels take (65536 positions, no padding): forward and dQ on windows
+    of queries against the oracle, and two sums over the whole row that need no oracle:
+    sum_j dV_j = sum over the group's heads and all queries of dO (each softmax row sums to 1)
+    and sum_j dK_j = 0 (each row of dS sums to 0)."""
+    print("attention S=65536", flush=True)
+    S, Hq, Hkv, D = 65536, 4, 2, 64
+    q, k, v = make_qkv(91, S, Hq, Hkv, D)
+    g = torch.Generator().manual_seed(92)
+    d_out = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16)
+    group, parent = synthetic.packed_row_ids(93, S, 16, 256, 4, 960)   # 16 * 4096 = 65536
+    plan = ops.attn_plan(group.to(gpu), parent.to(gpu))
+    qd, kd, vd = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.attn_fwd(qd, kd, vd, plan)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, out, lse, d_out.to(gpu), plan)
+    out_c, lse_c, dq_c = out.float().cpu(), lse.cpu(), dq.float().cpu()
+    for start in (0, 4096 - 32, 32768 + 256 + 960 - 8, S - 64):
+        rows = torch.arange(start, start + 64)
+        qw = q.float().clone().requires_grad_(True)
+        ref_out, ref_lse = attn_oracle.attention_rows(qw, k, v, group, parent, rows)
+        ref_out.backward(d_out[rows].float())
+        assert (lse_c[:, rows] - ref_lse.detach()).abs().max().item() <= 2e-3
+        assert rel_l2(out_c[rows], ref_out.detach()) <= 1e-2
+        assert rel_l2(dq_c[rows], qw.grad[rows]) <= 1e-2
+    rep = Hq // Hkv
+    want_dv = d_out.double().view(S, Hkv, rep, D).sum((0, 2))            # [Hkv, D]
+    got_dv = dv.double().cpu().sum(0)
+    assert ((got_dv - want_dv).norm() / want_dv.norm()).item() <= 1e-2
+    # rounding only: bf16 stores of 65536 rows, each about |dK_j| * 2^-9
+    dk64 = dk.double().cpu()
+    assert dk64.sum(0).abs().max().item() <= 2.0 ** -8 * dk64.abs().sum(0).max().item()
+
+
 def test_attn_bwd_mixed_light_and_heavy_key_blocks(artk_lib, gpu):
     """Grouped-query backward where early key blocks are seen by many (tile, head)
     pairs (one work-group per head, fp32 partials, reduction) and late ones by few
