@@ -81,6 +81,19 @@ def test_lora_config2_full_size(artk_lib, gpu, n_out):
     assert rel_l2(dB, dB0) <= TOL
 
 
+def test_lora_down_projection_full_size(artk_lib, gpu):
+    """The seventh target module of the reference's adapter config (down_proj, 11008 -> 2048,
+    src/art/dev/model.py:54-62) at full size, with rank 16."""
+    print("lora down_proj 11008 -> 2048, r=16", flush=True)
+    x, W, A, B, up = make(4096, 11008, 2048, 16, 1717)
+    y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, 1.0, up)
+    y, dx, dA, dB = run_gpu(x, W, A, B, up, 1.0, gpu)
+    assert rel_l2(y, y0) <= TOL
+    assert rel_l2(dx, dx0) <= TOL
+    assert rel_l2(dA, dA0) <= TOL
+    assert rel_l2(dB, dB0) <= TOL
+
+
 def test_lora_module_autograd(artk_lib, gpu):
     torch.manual_seed(0)
     mod = LoRALinear(256, 320, r=8, lora_alpha=16, device=gpu, dtype=torch.float32)
