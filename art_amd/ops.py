@@ -55,6 +55,7 @@ def _mask_u8(mask: torch.Tensor) -> torch.Tensor:
 # transposed copies of frozen weights
 # -----------------------------------------------------------------------------
 _transpose_cache: "dict[int, tuple]" = {}
+_frozen_cache: "dict[int, tuple]" = {}
 
 
 def transpose(x: torch.Tensor) -> torch.Tensor:
@@ -85,6 +86,29 @@ def transposed_weight(w: torch.Tensor) -> torch.Tensor:
         return wt
     _transpose_cache[key] = (ref, w._version, w.data_ptr(), wt)
     return wt
+
+
+def frozen_bf16(w: torch.Tensor) -> torch.Tensor:
+    """A detached bf16 view (or copy, if ``w`` has another dtype) of a frozen weight that is
+    the *same tensor object* from call to call for as long as ``w`` is not modified in place,
+    so that per-weight caches keyed by the object (``transposed_weight``) keep hitting when a
+    caller starts from ``module.weight`` in every step."""
+    key = id(w)
+    hit = _frozen_cache.get(key)
+    if hit is not None:
+        ref, version, ptr, out = hit
+        if ref() is w and version == w._version and ptr == w.data_ptr():
+            return out
+    out = w.detach()
+    if out.dtype != torch.bfloat16:
+        out = out.to(torch.bfloat16)
+    out = out.contiguous()
+    try:
+        ref = weakref.ref(w, lambda _r, k=key: _frozen_cache.pop(k, None))
+    except TypeError:  # pragma: no cover
+        return out
+    _frozen_cache[key] = (ref, w._version, w.data_ptr(), out)
+    return out
 
 
 def gemm_nt(p: torch.Tensor, q: torch.Tensor, out_f32: bool = False) -> torch.Tensor:

@@ -66,9 +66,16 @@ class _LogprobFn(torch.autograd.Function):
 
 
 def _as_vh(lm_head_t: torch.Tensor) -> torch.Tensor:
-    """The [V, H] row-major weight behind the reference's ``lm_head_t`` ([H, V] view)."""
-    w = lm_head_t.t()
-    return w if w.is_contiguous() else w.contiguous()
+    """The bf16 [V, H] row-major weight behind the reference's ``lm_head_t`` ([H, V] view).
+    When the view was made from the weight itself (``weight.t()``, as the reference does,
+    src/art/local/train.py:76-78), the same tensor object comes back in every step, so the
+    cached transposed copy of the weight is found again."""
+    H, V = lm_head_t.shape
+    base = lm_head_t._base
+    if (base is not None and base.dim() == 2 and tuple(base.shape) == (V, H) and base.is_contiguous()
+            and base.data_ptr() == lm_head_t.data_ptr() and lm_head_t.stride() == (1, H)):
+        return ops.frozen_bf16(base)
+    return lm_head_t.t().contiguous().to(torch.bfloat16)
 
 
 def _calculate_logprobs(
@@ -87,7 +94,7 @@ def _calculate_logprobs(
         seq_len % chunk_size == 0
     ), f"Sequence length ({seq_len}) must be evenly divisible by chunk size ({chunk_size})"
     hidden = hidden_states.to(torch.bfloat16).contiguous()
-    lm_head = _as_vh(lm_head_t).to(torch.bfloat16)
+    lm_head = _as_vh(lm_head_t)
     ids = next_input_ids.contiguous()
     return _LogprobFn.apply(hidden, lm_head, ids, ops.DEFAULT_CHUNK_TOKENS)
 
@@ -259,7 +266,7 @@ def get_compute_loss_fn(trainer) -> Callable[..., torch.Tensor]:
         epsilon = _config.get("epsilon", 0.2)
         epsilon_high = _config.get("epsilon_high", epsilon)
         loss, metrics, _ = fused_grpo_loss(
-            hidden_states, lm_head.detach().to(torch.bfloat16), inputs["tokens"], inputs["logprobs"],
+            hidden_states, ops.frozen_bf16(lm_head), inputs["tokens"], inputs["logprobs"],
             inputs["advantages"], inputs["assistant_mask"], inputs["weights"], epsilon, epsilon_high,
             ref_logprobs, config.beta, skip_inactive=True)  # new_logprobs are not used here
 

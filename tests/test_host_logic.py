@@ -101,3 +101,21 @@ def test_wrappers_refuse_cpu_tensors():
         ops.logprob_fwd(h, w, torch.zeros(4, dtype=torch.int64), False, 4)
     with pytest.raises(ValueError, match="no CPU path"):
         ops.transpose(h)
+
+
+def test_frozen_weight_view_is_stable_until_the_weight_changes():
+    """``weight.t()`` is a new view object in every step; the wrapper maps it back to one
+    detached bf16 tensor per weight version, so caches keyed by the tensor object hit."""
+    from art_amd.train import _as_vh
+    w = torch.nn.Parameter(torch.randn(12, 4).to(torch.bfloat16), requires_grad=False)
+    a, b = _as_vh(w.t()), _as_vh(w.t())
+    assert a is b and a.data_ptr() == w.data_ptr() and a.shape == (12, 4)
+    with torch.no_grad():
+        w.add_(1)
+    c = _as_vh(w.t())
+    assert c is not a and torch.equal(c, w)
+    w32 = torch.nn.Parameter(torch.randn(12, 4), requires_grad=False)
+    d = _as_vh(w32.t())
+    assert d is _as_vh(w32.t()) and d.dtype == torch.bfloat16
+    plain = torch.randn(4, 12).to(torch.bfloat16)      # an [H, V] tensor that is not such a view
+    assert torch.equal(_as_vh(plain), plain.t())
