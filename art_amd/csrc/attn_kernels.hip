@@ -209,8 +209,15 @@ struct AttnTile {
   static constexpr int BYTES = 64 * ROW;
   static constexpr int N8 = BYTES / 1024 / 8;          // DMA instructions per wave, 8 waves
   static constexpr int N4 = BYTES / 1024 / 4;          // 4 waves
+  // XOR applied to the chunk index of a row.  Two access patterns must be free of
+  // bank conflicts (256 bytes = 16 chunk slots per bank line; with D = 64 two rows
+  // share a line): a row-fragment read takes one chunk of 16 consecutive rows, a
+  // transposed read takes 4 consecutive chunks (aligned to 4) of 4 consecutive
+  // rows (aligned to 4).  So rows that differ in their low bits must land in
+  // different aligned groups of 4 chunks, and the 16 rows of a fragment read in 16
+  // different slots: the low row bits go to the high chunk bits and vice versa.
   __device__ static __forceinline__ int swz(int row) {
-    return CHK == 16 ? (row & 15) : ((row >> 1) & 7);
+    return CHK == 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
   }
   // per-lane byte offset (global side) of DMA instruction `instr` of a tile whose
   // rows are `stride` elements apart
