@@ -253,12 +253,22 @@ __global__ __launch_bounds__(256) void lse_finalize_kernel(const float2* __restr
   const int n = rows.n();
   float m = -INFINITY, l = 0.f;
   if (t < n) {
-    for (int i = sl; i < nparts; i += 16) {
-      const float2 v = part[(int64_t)i * Tc + t];
-      const float mn = fmaxf(m, v.x);
-      if (mn != -INFINITY)
-        l = l * __builtin_amdgcn_exp2f((m - mn) * LOG2E) + v.y * __builtin_amdgcn_exp2f((v.x - mn) * LOG2E);
-      m = mn;
+    // eight loads in flight per thread (the merge itself is a dependent chain), same merge order
+    for (int i0 = sl; i0 < nparts; i0 += 16 * 8) {
+      float2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + 16 * u;
+        v[u] = i < nparts ? part[(int64_t)i * Tc + t] : make_float2(-INFINITY, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (i0 + 16 * u >= nparts) break;
+        const float mn = fmaxf(m, v[u].x);
+        if (mn != -INFINITY)
+          l = l * __builtin_amdgcn_exp2f((m - mn) * LOG2E) + v[u].y * __builtin_amdgcn_exp2f((v[u].x - mn) * LOG2E);
+        m = mn;
+      }
     }
   }
   red[sl][tl] = make_float2(m, l);
