@@ -50,9 +50,10 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(case, sample_tokens: int):
+def cpu_baseline(case, sample_tokens: int, gpu_logprob=None, gpu_d_hidden=None, mask_count=None):
     """CPU oracle (fp32, autograd w.r.t. hidden) on the first `sample_tokens`
-    positions of the same case; tokens/s on the host cores."""
+    positions of the same case; tokens/s on the host cores.  With the GPU results of the
+    whole batch given, the same oracle run doubles as the parity check of this run."""
     import torch
 
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -64,9 +65,9 @@ def cpu_baseline(case, sample_tokens: int):
             sl(case.assistant_mask), sl(case.weights))
     chunk = 256 if n % 256 == 0 else n
     t0 = time.perf_counter()
-    grpo_oracle.loss_and_grad(*args, chunk_size=chunk)
+    ref = grpo_oracle.loss_and_grad(*args, chunk_size=chunk)
     dt = time.perf_counter() - t0
-    return {
+    out = {
         "value": n / dt,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
@@ -74,6 +75,31 @@ def cpu_baseline(case, sample_tokens: int):
         "sample": f"first {n} of {case.hidden.shape[1]} positions, full vocab, fp32 torch-CPU oracle "
                   f"fwd+bwd, 1 run of {dt:.1f} s",
     }
+    parity = None
+    if gpu_logprob is not None and n > 1:
+        # Every position's logprob and d_hidden row depend on the rest of the batch only through
+        # the loss denominator (mask count + 1e-6); the last position of the sample is left out
+        # (its target lies outside the sample).
+        m_sample = float(grpo_oracle.shift_tensor(sl(case.assistant_mask), False).sum())
+        scale = (m_sample + 1e-6) / (float(mask_count) + 1e-6)
+        lp_err = (gpu_logprob[: n - 1].float().cpu() - ref["logprobs"][0, : n - 1]).abs().max().item()
+        want = ref["d_hidden"][0, : n - 1].double() * scale
+        got = gpu_d_hidden[: n - 1].double().cpu()
+        parity = {"positions": n - 1, "logprob_max_abs_err": lp_err,
+                  "d_hidden_rel_l2": ((got - want).norm() / want.norm()).item(),
+                  "tolerances": {"logprob_max_abs_err": 2e-3, "d_hidden_rel_l2": 1e-2}}
+    return out, parity
+
+
+def input_digests(case):
+    """SHA-256 (first 16 hex digits) of the integer and boolean inputs of a case."""
+    import hashlib
+
+    import numpy as np
+
+    arrays = {"tokens": case.tokens.numpy(), "assistant_mask": case.assistant_mask.numpy().astype(np.uint8),
+              "traj_id": case.traj_id.numpy(), "group_of_traj": np.asarray(case.group_of_traj)}
+    return {k: hashlib.sha256(np.ascontiguousarray(v).tobytes()).hexdigest()[:16] for k, v in arrays.items()}
 
 
 def timed(fn, steps, warmup):
@@ -826,8 +852,11 @@ def main():
     if torch_ms is not None:
         result["torch_gpu_same_algorithm"] = {"value": T / (torch_ms * 1e-3), "unit": "tokens/s",
                                               "ms_per_step": torch_ms, "note": torch_note}
+    result["config"]["input_sha256"] = input_digests(case)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(case, args.cpu_sample_tokens)
+        result["cpu_baseline"], parity = cpu_baseline(case, args.cpu_sample_tokens, out[1], out[2], mask_count)
+        if parity:
+            result["parity_same_run"] = parity
     print(json.dumps(result))
 
 
