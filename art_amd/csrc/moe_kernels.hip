@@ -584,6 +584,12 @@ int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const vo
                  "null pointer argument");
   ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(A) && aligned16(B) && aligned16(y),
                  "pointers must be 16-byte aligned");
+  // gathered rows are addressed with 31-bit byte offsets from x; gather[i] < n_rows
+  if (gather != nullptr && n_rows * in * 2 >= (1ll << 31)) {
+    set_error("with a row gather, n_rows * in * 2 bytes (%lld) must stay below 2 GiB",
+              (long long)(n_rows * in * 2));
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
   uint16_t* xa16 = ws.take<uint16_t>((size_t)n_rows * RP);

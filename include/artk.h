@@ -186,7 +186,8 @@ int32_t artk_moe_route(const float* router_logits, int64_t T, int32_t E, int32_t
  *   y[i,:] = x[src(i),:] W_e^T + scale (x[src(i),:] A_e^T) B_e^T,  e = expert of row i
  *   src(i) = gather[i] when gather != NULL (rows of x picked by row_token), else i.
  *   W bf16 [E,out,in], A bf16 [E,r,in], B bf16 [E,out,r]
- *   y bf16 [n_rows,out] out, xa f32 [n_rows,r] out (kept for the backward) */
+ *   y bf16 [n_rows,out] out, xa f32 [n_rows,r] out (kept for the backward)
+ *   With a gather, n_rows * in * 2 bytes must stay below 2 GiB (31-bit offsets from x). */
 size_t artk_moe_lora_grouped_fwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
                                                  int32_t r);
 int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const void* W, const void* A,

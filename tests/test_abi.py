@@ -45,6 +45,14 @@ def test_argument_errors_have_codes_and_messages(artk_lib):
     assert rc == _lib.ERR_INVALID_ARGUMENT  # clip_lo > clip_hi
     rc = artk_lib.artk_lora_linear_fwd(p, p, p, p, 2.0, 64, 64, 64, 5, p, p, p, 4096, None)  # rank 5
     assert rc == _lib.ERR_UNSUPPORTED_SHAPE
+    # gathered MoE rows further than 2 GiB from x
+    rc = artk_lib.artk_moe_lora_grouped_fwd(p, p, p, p, p, 2.0, p, p, p, 1 << 20, 4096, 64, 8, 8, p, p, p, 4096, None)
+    assert rc == _lib.ERR_UNSUPPORTED_SHAPE and b"2 GiB" in artk_lib.artk_last_error()
+    # attention: row length not a multiple of 256, head dimension 96
+    rc = artk_lib.artk_attn_plan(p, p, 1000, p, 1 << 20, None)
+    assert rc == _lib.ERR_UNSUPPORTED_SHAPE
+    rc = artk_lib.artk_attn_fwd(p, p, p, p, 256, 2, 1, 96, 192, 96, 96, 96, 96, 96, 192, 96, 0.1, p, p, p, 4096, None)
+    assert rc == _lib.ERR_UNSUPPORTED_SHAPE and b"head dimension" in artk_lib.artk_last_error()
 
 
 def test_check_raises(artk_lib):
