@@ -399,12 +399,27 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
     floatx16 sc[2];
 #pragma unroll
     for (int j = 0; j < 16; ++j) sc[0][j] = sc[1][j] = 0.f;
+    {
+      // K fragments three steps ahead of the MFMAs that use them (LDS latency)
+      constexpr int NS = D / 16, PF = 3;
+      bf16x8 kf[NS][2];
 #pragma unroll
-    for (int s = 0; s < D / 16; ++s) {
+      for (int s = 0; s < PF; ++s) {
+        kf[s][0] = T::row_frag(st, n, s, h);
+        kf[s][1] = T::row_frag(st, 32 + n, s, h);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF, 0);
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-        sc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::row_frag(st, 32 * kt + n, s, h), qf[s], sc[kt],
-                                                         0, 0, 0);
+      for (int s = 0; s < NS; ++s) {
+        if (s + PF < NS) {
+          kf[s + PF][0] = T::row_frag(st, n, s + PF, h);
+          kf[s + PF][1] = T::row_frag(st, 32 + n, s + PF, h);
+        }
+        sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s][0], qf[s], sc[0], 0, 0, 0);
+        sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s][1], qf[s], sc[1], 0, 0, 0);
+        if (s + PF < NS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      }
     }
 
     // scale, mask, running max
