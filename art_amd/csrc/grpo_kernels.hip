@@ -987,6 +987,24 @@ static int64_t clamp_chunk(int64_t T, int64_t V, int64_t chunk_tokens) {
   return chunk_tokens;
 }
 
+// Lengths of the chunks of a batch of T positions with at most Tc per chunk.  When Tc is
+// a whole number of tiles the tiles are spread evenly over the chunks (16384 positions, Tc
+// = 5632: 22 + 21 + 21 tiles rather than 22 + 22 + 20), which wastes less of the last round
+// of work-groups of each forward launch.
+struct ChunkSteps {
+  int64_t Tc, base, extra;
+  bool balanced;
+  ChunkSteps(int64_t T, int64_t Tc_, bool allow) : Tc(Tc_), base(0), extra(0), balanced(false) {
+    if (allow && Tc % TILE == 0) {
+      const int64_t nchunks = (T + Tc - 1) / Tc, tiles = (T + TILE - 1) / TILE;
+      base = tiles / nchunks;
+      extra = tiles % nchunks;
+      balanced = true;
+    }
+  }
+  int64_t step(int64_t chunk) const { return balanced ? (base + (chunk < extra ? 1 : 0)) * TILE : Tc; }
+};
+
 size_t artk_logprob_bwd_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {
   Workspace ws(nullptr, 0);
   ChunkScratch c;
@@ -1013,9 +1031,12 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
-    const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
-    // The scratch row pitch is V, so a shorter last chunk simply uses fewer rows.
+  const ChunkSteps steps(T, Tc, true);
+  int64_t step = 0;
+  for (int64_t t0 = 0, ci = 0; t0 < T; t0 += step, ++ci) {
+    step = steps.step(ci);
+    const int64_t n = (T - t0 < step) ? (T - t0) : step;
+    // The scratch row pitch is V, so a shorter chunk simply uses fewer rows.
     need_from_grad_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(grad_logprob + t0, n, c.need);
     ARTK_CHECK_LAUNCH();
     const ChunkRows rows = dense_rows(t0, n);
@@ -1140,7 +1161,10 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
   }
   // In skip mode the number of evaluated rows is known only on the device: every
   // chunk the worst case needs is launched and the ones past the end do nothing.
-  for (int64_t t0 = 0; t0 < T; t0 += Tc) {
+  const ChunkSteps steps(T, Tc, !skip);
+  int64_t step = 0;
+  for (int64_t t0 = 0, ci = 0; t0 < T; t0 += step, ++ci) {
+    step = steps.step(ci);
     ChunkRows rows;
     if (skip) {
       rows.row_token = c.eval_idx + t0;
@@ -1149,7 +1173,7 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
       rows.c0 = (int)t0;
       rows.cap = (int)Tc;
     } else {
-      const int64_t n = (T - t0 < Tc) ? (T - t0) : Tc;
+      const int64_t n = (T - t0 < step) ? (T - t0) : step;
       rows = dense_rows(t0, n);
       need_from_inputs_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(mask, weights, advantages,
                                                                            ref, t0, n, S, 1, c.need);
