@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None until
 # measured for the workload.  Source: profiles/lmhead_fwd_c3_pmc.md
-TRAFFIC_BYTES = {"c3": 1.80e10, "c1": None}
+TRAFFIC_BYTES = {"c3": 2.05e10, "c1": None}
 
 
 def parse():
