@@ -5,6 +5,8 @@ import ctypes as C
 import os
 import re
 
+import pytest
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -72,3 +74,19 @@ def test_workspace_sizes_are_monotone(artk_lib):
     c = artk_lib.artk_grpo_fused_workspace_bytes(16384, 152064, 3584, 2048)
     assert 0 < c < b and a <= b
     assert artk_lib.artk_logprob_fwd_workspace_bytes(16384, 152064, 3584) > 16384 * 1188 * 8
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/artk.h is the C-ABI: it must compile as C99 without any C++ or HIP header."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler here")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "artk.h"\nint main(void) { return (int)artk_abi_version(); }\n')
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, "-fsyntax-only",
+                        str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
