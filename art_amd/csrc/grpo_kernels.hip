@@ -1058,25 +1058,24 @@ size_t artk_grpo_loss_workspace_bytes(int64_t T) {
   return ws.used + 256;
 }
 
-int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const float* advantages,
-                       const uint8_t* mask, const float* weights, const float* ref_logprob,
-                       int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi, float beta,
-                       float* scalars, float* coef, void* workspace, size_t workspace_bytes,
-                       artk_stream_t stream) {
+// Shared body of artk_grpo_loss and artk_grpo_loss_static: the scratch (two f32 [T]
+// arrays of per-token terms and the mask count) is carved out of `ws`.
+static int32_t grpo_loss_run(const float* new_logprob, const float* old_logprob, const float* advantages,
+                             const uint8_t* mask, const float* weights, const float* ref_logprob,
+                             int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi, float beta,
+                             float* scalars, float* coef, Workspace& ws, hipStream_t st) {
   ARTK_CHECK_ARG(new_logprob && old_logprob && advantages && mask && weights && scalars,
                  "null pointer argument");
   ARTK_CHECK_ARG(T > 0 && S > 0 && T % S == 0 && T < (1ll << 31), "T must be a positive multiple of S below 2^31");
   ARTK_CHECK_ARG(shift == 0 || shift == 1, "shift must be 0 or 1");
   ARTK_CHECK_ARG(clip_lo <= clip_hi, "clip_lo must not exceed clip_hi");
-  Workspace ws(workspace, workspace_bytes);
   float* pl = ws.take<float>((size_t)T);
   float* kl = ws.take<float>((size_t)T);
   int* count = ws.take<int>(64);
   if (!ws.ok()) {
-    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, ws.size);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
-  hipStream_t st = (hipStream_t)stream;
   mask_count_kernel<<<1, 1024, 0, st>>>(mask, T, S, shift, count);
   ARTK_CHECK_LAUNCH();
   LossParams p;
@@ -1101,6 +1100,16 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
   grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, p.ref_lp ? beta : 0.f, scalars);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
+}
+
+int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const float* advantages,
+                       const uint8_t* mask, const float* weights, const float* ref_logprob,
+                       int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi, float beta,
+                       float* scalars, float* coef, void* workspace, size_t workspace_bytes,
+                       artk_stream_t stream) {
+  Workspace ws(workspace, workspace_bytes);
+  return grpo_loss_run(new_logprob, old_logprob, advantages, mask, weights, ref_logprob, shift, T, S,
+                       clip_lo, clip_hi, beta, scalars, coef, ws, (hipStream_t)stream);
 }
 
 size_t artk_grpo_fused_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens) {

@@ -31,11 +31,16 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
+  // NaN counts as -inf, so the order below is total: decreasing value, ties (also
+  // among -inf) to the lower expert index; every round picks an index in [0, E).
   float x[4];
+  unsigned taken = 0;  // bit i: element i of this lane is selected or past E
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int e = lane + 64 * i;
-    x[i] = e < E ? logits[t * E + e] : -INFINITY;
+    float v = e < E ? logits[t * E + e] : -INFINITY;
+    x[i] = v == v ? v : -INFINITY;
+    if (e >= E) taken |= 1u << i;
   }
   float m = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
   m = wave_max(m);
@@ -46,7 +51,7 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
     int bi = 0x7fffffff;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (x[i] > bv) {
+      if (!(taken >> i & 1) && (bi == 0x7fffffff || x[i] > bv)) {
         bv = x[i];
         bi = lane + 64 * i;
       }
@@ -54,20 +59,21 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__
     for (int o = 32; o > 0; o >>= 1) {
       const float ov = __shfl_xor(bv, o, 64);
       const int oi = __shfl_xor(bi, o, 64);
-      if (ov > bv || (ov == bv && oi < bi)) {
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
         bv = ov;
         bi = oi;
       }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (lane + 64 * i == bi) x[i] = -INFINITY;
-    const float pj = expf(bv - m);
+      if (lane + 64 * i == bi) taken |= 1u << i;
+    // exp(-inf - m) = 0; a row without any finite logit (m = -inf) has no mass at all
+    const float pj = bv == -INFINITY ? 0.f : expf(bv - m);
     psum += pj;
     if (lane == j) myp = pj;
     if (lane == 0) topk_idx[t * k + j] = bi;
   }
-  if (lane < k) topk_w[t * k + lane] = myp / psum;
+  if (lane < k) topk_w[t * k + lane] = psum > 0.f ? myp / psum : 0.f;
 }
 
 // ----------------------------------------------------------------------------
@@ -81,7 +87,8 @@ __global__ __launch_bounds__(PERM_CHUNK) void moe_hist_kernel(const int* __restr
   for (int i = threadIdx.x; i < E; i += PERM_CHUNK) hist[i] = 0;
   __syncthreads();
   const int f = blockIdx.x * PERM_CHUNK + threadIdx.x;
-  if (f < n) atomicAdd(&hist[keys[f]], 1);
+  // keys come from moe_topk_kernel and lie in [0, E); anything else is ignored
+  if (f < n && (unsigned)keys[f] < (unsigned)E) atomicAdd(&hist[keys[f]], 1);
   __syncthreads();
   for (int i = threadIdx.x; i < E; i += PERM_CHUNK) cnt[blockIdx.x * E + i] = hist[i];
 }
@@ -146,7 +153,8 @@ __global__ __launch_bounds__(PERM_CHUNK) void moe_scatter_kernel(const int* __re
   for (int i = threadIdx.x; i < NW * 256; i += PERM_CHUNK) (&hist[0][0])[i] = 0;
   __syncthreads();
   const int f = blockIdx.x * PERM_CHUNK + threadIdx.x;
-  const int key = f < n ? keys[f] : -1;
+  int key = f < n ? keys[f] : -1;
+  if ((unsigned)key >= (unsigned)E) key = -1;  // never produced by moe_topk_kernel
   if (key >= 0) atomicAdd(&hist[wave][key], 1);
   int rank = 0;
   for (int j = 0; j < 64; ++j) {
@@ -154,7 +162,7 @@ __global__ __launch_bounds__(PERM_CHUNK) void moe_scatter_kernel(const int* __re
     rank += (j < lane && kj == key) ? 1 : 0;
   }
   __syncthreads();
-  if (f < n) {
+  if (key >= 0) {
     for (int w = 0; w < wave; ++w) rank += hist[w][key];
     const int pos = base[blockIdx.x * E + key] + rank;
     perm[pos] = f;

@@ -552,3 +552,28 @@ def profile_collect(kind: int) -> Tuple[float, int]:
     ms, n = C.c_double(0.0), C.c_int64(0)
     _lib.check(_lib.load().artk_profile_collect(kind, C.byref(ms), C.byref(n)))
     return ms.value, n.value
+
+
+# -----------------------------------------------------------------------------
+# ceilings of the part (measurement aids)
+# -----------------------------------------------------------------------------
+def mfma_loop(operands: torch.Tensor, iters: int, blocks: int, sink: Optional[torch.Tensor] = None) -> float:
+    """Launches the MFMA-only loop; returns the flop it executes (time it with events)."""
+    _need(operands, "operands", torch.bfloat16)
+    if sink is None:
+        sink = torch.empty(blocks * 512, dtype=torch.float32, device=operands.device)
+    _need(sink, "sink", torch.float32, (blocks * 512,))
+    _lib.check(_lib.load().artk_mfma_loop(operands.data_ptr(), operands.numel(), int(iters), int(blocks),
+                                          sink.data_ptr(), _stream(operands.device)))
+    return float(blocks) * 8 * iters * 32 * 32768.0
+
+
+def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> int:
+    """dst = src with the library's plain copy kernel; returns the bytes copied."""
+    if not (src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("src and dst must be contiguous GPU tensors")
+    nbytes = src.numel() * src.element_size()
+    if nbytes != dst.numel() * dst.element_size():
+        raise ValueError("src and dst differ in size")
+    _lib.check(_lib.load().artk_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream(src.device)))
+    return nbytes

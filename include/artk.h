@@ -167,8 +167,11 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
  *
  * artk_moe_route: top-k experts per token and the expert-contiguous permutation.
  *   router_logits f32 [T,E]
- *   topk_idx i32 [T,k]   experts by decreasing logit, ties to the lower index
- *   topk_w   f32 [T,k]   softmax probabilities of the chosen experts, renormalised
+ *   topk_idx i32 [T,k]   experts by decreasing logit, ties to the lower index; a NaN
+ *                        logit counts as -inf, so every index lies in [0,E) whatever the
+ *                        row holds (ties among -inf also go to the lower index)
+ *   topk_w   f32 [T,k]   softmax probabilities of the chosen experts, renormalised; an
+ *                        expert at -inf gets 0, a row without any finite logit all 0
  *   perm     i32 [T*k]   perm[i] = flat (token*k + slot) index of sorted row i;
  *                        stable sort of the token-major list by expert id
  *   inv_perm i32 [T*k]   inverse of perm;  row_token i32 [T*k] = perm[i] / k
@@ -304,6 +307,21 @@ int32_t artk_nf4_dequant(const void* packed, const float* absmax, const void* ab
 #define ARTK_PROF_ATTN_BWD_Q 7
 int32_t artk_profile_enable(int32_t on);
 int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches);
+
+/* ------------------------------------------------------------------------- *
+ * Ceilings of the part, measured rather than quoted (measurement aids; no
+ * counterpart in the reference).
+ * artk_mfma_loop: `blocks` work-groups of 8 waves; every wave keeps the register
+ *   tile of the GEMM main loop (4 x 2 MFMA 32x32x16 bf16 tiles) and issues
+ *   `iters` rounds of 32 MFMAs on fragments read once from `operands`
+ *   (bf16 [n_operands], n_operands >= 4096, a multiple of 8); no LDS, no memory
+ *   traffic inside the loop.  Work: blocks * 8 * iters * 32 * 32768 flop.
+ *   sink f32 [blocks * 512] receives a checksum per lane.
+ * artk_stream_copy: dst[i] = src[i], 16 bytes per lane and step (bytes % 16 == 0).
+ * ------------------------------------------------------------------------- */
+int32_t artk_mfma_loop(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
+                       float* sink, artk_stream_t stream);
+int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -5,7 +5,9 @@ restate: PARITY UNPINNED against the reference.  The contract is the benchmark
 configuration plus the usual definitions, stated here with plain torch:
   routing      softmax over router logits in fp32, top-k, renormalise (the
                semantics of transformers' Qwen3-MoE block); selection on the
-               logits, ties to the lower expert index
+               logits, ties to the lower expert index; a NaN logit counts as
+               -inf, an expert at -inf gets weight 0, a row without a finite
+               logit gets weights 0
   permutation  stable sort of the token-major (token, slot) list by expert id
   projections  per expert y = x W_e^T + scale (x A_e^T) B_e^T  (Python loop)
 Pinned in tests/test_oracle_moe.py by brute force on tiny inputs, by
@@ -20,11 +22,17 @@ def route(router_logits: torch.Tensor, k: int):
     """Returns dict(topk_idx [T,k], topk_w [T,k], perm [T*k], inv_perm, row_token, offsets [E+1])."""
     T, E = router_logits.shape
     logits = router_logits.float()
-    probs = torch.softmax(logits, dim=-1)
+    # NaN counts as -inf (a masked expert); the order is then total
+    logits = torch.where(torch.isnan(logits), torch.full_like(logits, float("-inf")), logits)
     order = torch.sort(-logits, dim=-1, stable=True).indices  # ties -> lower index first
     topk_idx = order[:, :k]
-    p = probs.gather(-1, topk_idx)
-    topk_w = p / p.sum(-1, keepdim=True)
+    # softmax mass of the chosen experts; exp(-inf - m) = 0, and a row without any finite
+    # logit carries no mass at all (its weights are 0 rather than NaN)
+    m = logits.max(-1, keepdim=True).values
+    chosen = logits.gather(-1, topk_idx)
+    p = torch.where(torch.isinf(chosen) & (chosen < 0), torch.zeros_like(chosen), torch.exp(chosen - m))
+    tot = p.sum(-1, keepdim=True)
+    topk_w = torch.where(tot > 0, p / tot, torch.zeros_like(p))
     flat = topk_idx.reshape(-1)
     perm = torch.sort(flat, stable=True).indices
     inv_perm = torch.empty_like(perm)

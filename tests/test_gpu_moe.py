@@ -50,6 +50,33 @@ def test_route_ties_and_empty_experts(artk_lib, gpu):
     assert (r.offsets.cpu()[4:9] == r.offsets.cpu()[4]).all()  # experts 3..8 empty
 
 
+def test_route_nan_and_masked_logits(artk_lib, gpu):
+    """Rows that are all NaN, or have fewer than k logits above -inf (masked experts, a diverged
+    router), still give expert indices in [0, E): NaN counts as -inf, ties go to the lower index."""
+    print("moe route with NaN / -inf rows", flush=True)
+    g = torch.Generator().manual_seed(5)
+    T, E, k = 517, 128, 8
+    logits = torch.randn(T, E, generator=g)
+    logits[3] = float("nan")
+    logits[7] = float("-inf")
+    logits[11, 5:] = float("-inf")               # 5 finite logits, k = 8
+    logits[12, ::3] = float("nan")
+    logits[13, :] = float("-inf")
+    logits[13, 100] = 0.25                       # one finite logit
+    logits[200:260, 64:] = float("-inf")         # half of the experts masked
+    r, ref = check_routing(logits, k, gpu)
+    idx = r.topk_idx.cpu()
+    assert int(idx.min()) >= 0 and int(idx.max()) < E
+    assert idx[3].tolist() == list(range(8)) and r.topk_w.cpu()[3].abs().max().item() == 0.0
+    assert idx[13, 0].item() == 100 and r.topk_w.cpu()[13].tolist() == [1.0] + [0.0] * 7
+    assert not torch.isnan(r.topk_w.cpu()).any()
+    # one lane group past E (E = 200 leaves lanes of the fourth group without an expert)
+    logits = torch.randn(64, 200, generator=g)
+    logits[5] = float("nan")
+    logits[6, 3:] = float("-inf")
+    check_routing(logits, 5, gpu)
+
+
 def make_experts(E, n_out, n_in, r, seed):
     g = torch.Generator().manual_seed(seed)
     W = (0.02 * torch.randn(E, n_out, n_in, generator=g)).to(torch.bfloat16)

@@ -24,6 +24,23 @@ def test_route_brute_force_with_ties():
     assert r["row_token"].tolist() == [1, 2, 0, 1, 0, 2]
 
 
+def test_route_nan_and_masked_rows():
+    """NaN counts as -inf; ties among -inf go to the lower index; weights of -inf experts are 0,
+    and a row without any finite logit has all weights 0 (hand-computed)."""
+    ninf, nan = float("-inf"), float("nan")
+    logits = torch.tensor([[nan, nan, nan, nan],          # nothing finite: experts 0, 1
+                           [ninf, 2.0, ninf, ninf],       # one finite: expert 1, then 0
+                           [1.0, nan, 1.0, 3.0],          # 3, then the tie 0 < 2
+                           [ninf, ninf, 0.0, 0.0]])       # 2, 3
+    r = M.route(logits, 2)
+    assert r["topk_idx"].tolist() == [[0, 1], [1, 0], [3, 0], [2, 3]]
+    e2 = 1.0 / (1.0 + torch.exp(torch.tensor(-2.0)).item())
+    want = [[0.0, 0.0], [1.0, 0.0], [e2, 1.0 - e2], [0.5, 0.5]]
+    assert torch.allclose(r["topk_w"], torch.tensor(want), atol=1e-6)
+    assert 0 <= int(r["topk_idx"].min()) and int(r["topk_idx"].max()) < 4
+    assert sorted(r["perm"].tolist()) == list(range(8))
+
+
 def test_route_matches_topk_and_invariants():
     g = torch.Generator().manual_seed(0)
     T, E, k = 300, 16, 4
