@@ -65,6 +65,7 @@ SIGNATURES = {
     "artk_attn_bwd": (
         _i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i32, _i32, _i32, C.POINTER(_i64), _f32, _p, _p, _p, _p,
                _sz, _p]),
+    "artk_attn_bwd_tuning": (_i32, [_i32]),
     "artk_sumsq_f32_workspace_bytes": (_sz, []),
     "artk_sumsq_f32": (_i32, [_p, _i64, _p, _p, _sz, _p]),
     "artk_adamw_step": (_i32, [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _f32, _i32, _p, _f32, _p]),

@@ -968,6 +968,9 @@ __global__ __launch_bounds__(256) void attn_kv_reduce_kernel(const float* __rest
 
 }  // namespace artk
 
+// Threshold override of artk_attn_bwd_tuning for calls made on this thread (-1: automatic).
+static thread_local int g_light_max_override = -1;
+
 using namespace artk;
 
 extern "C" {
@@ -1171,8 +1174,7 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
       cus = 256;
     p.light_max = pl.nKb2 * Hkv >= cus ? ATT_LIGHT_MAX : 0;
-    // tuning / test knob: ARTK_ATTN_LIGHT_MAX=<n> forces the threshold
-    if (const char* e = getenv("ARTK_ATTN_LIGHT_MAX")) p.light_max = atoi(e);
+    if (g_light_max_override >= 0) p.light_max = g_light_max_override;  // artk_attn_bwd_tuning
   }
   prof_begin(PROF_ATTN_BWD_KV, st);
   if (D == 128)
@@ -1195,6 +1197,11 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
     attn_bwd_dq_kernel<64><<<(unsigned)(pl.nQb * Hq), 512, 0, st>>>(p);
   prof_end(PROF_ATTN_BWD_Q, st);
   ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_attn_bwd_tuning(int32_t light_max) {
+  g_light_max_override = light_max < 0 ? -1 : light_max;
   return ARTK_OK;
 }
 

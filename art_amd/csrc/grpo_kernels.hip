@@ -1058,7 +1058,7 @@ size_t artk_grpo_loss_workspace_bytes(int64_t T) {
   return ws.used + 256;
 }
 
-// Shared body of artk_grpo_loss and artk_grpo_loss_static: the scratch (two f32 [T]
+// Body of artk_grpo_loss: the scratch (two f32 [T]
 // arrays of per-token terms and the mask count) is carved out of `ws`.
 static int32_t grpo_loss_run(const float* new_logprob, const float* old_logprob, const float* advantages,
                              const uint8_t* mask, const float* weights, const float* ref_logprob,

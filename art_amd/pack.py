@@ -162,19 +162,74 @@ def packed_tensors_to_dir(tensors: PackedTensors, dir: str) -> dict:
 
 
 class RowStager:
-    """Moves one packed row at a time to the GPU through a reused pinned buffer
-    (allocated pinned: registering existing memory is not supported everywhere).
-    The training loop takes rows `[offset : offset + 1]` (src/art/local/service.py:96-104)."""
+    """Moves packed rows to the GPU one at a time, the way the training loop consumes them
+    (rows `[offset : offset + 1]`, src/art/local/service.py:96-104), with the copy of row i+1
+    overlapping the step on row i.
+
+    Two slots, each a set of pinned host buffers (allocated pinned: registering existing
+    memory is not supported everywhere) and a set of device buffers.  A row goes
+    file / host tensor -> pinned slot -> device slot on a copy stream of its own; the consumer's
+    stream waits for one event per row, and the copy stream waits for the event the consumer's
+    stream records when it is done with the slot, so nothing synchronises a whole stream or the
+    device.  The host only blocks when it wants to refill a pinned slot whose previous copy
+    (two rows ago) has not left yet."""
+
+    DEPTH = 2
 
     def __init__(self, sequence_length: int, device: torch.device):
-        self.device = device
-        self.pinned = {key: torch.empty((1, sequence_length), dtype=dtype).pin_memory()
-                       for key, dtype in DISK_DTYPES.items()}
+        self.device = torch.device(device)
+        self.copy_stream = torch.cuda.Stream(self.device)  # default priority
+        self.slots = []
+        for _ in range(self.DEPTH):
+            self.slots.append({
+                "pinned": {key: torch.empty((1, sequence_length), dtype=dtype).pin_memory()
+                           for key, dtype in DISK_DTYPES.items()},
+                "dev": {key: torch.empty((1, sequence_length), dtype=dtype, device=self.device)
+                        for key, dtype in DISK_DTYPES.items()},
+                "copied": torch.cuda.Event(),     # recorded on the copy stream after the H2D copies
+                "released": torch.cuda.Event(),   # recorded on the consumer's stream when it moves on
+                "in_flight": False,
+            })
+
+    def _stage(self, tensors: PackedTensors, row: int, slot: dict) -> None:
+        if slot["in_flight"]:
+            slot["copied"].synchronize()          # the pinned buffers are about to be overwritten
+        for key, buf in slot["pinned"].items():
+            buf.copy_(tensors[key][row:row + 1])
+        self.copy_stream.wait_event(slot["released"])   # no-op for an event never recorded
+        with torch.cuda.stream(self.copy_stream):
+            for key, buf in slot["pinned"].items():
+                slot["dev"][key].copy_(buf, non_blocking=True)
+            slot["copied"].record(self.copy_stream)
+        slot["in_flight"] = True
+
+    def rows(self, tensors: PackedTensors):
+        """Yields the rows of `tensors` (host tensors or the memory maps of
+        `packed_tensors_from_dir`) as dicts of device tensors [1, S].  A yielded dict stays
+        valid until the generator is advanced twice more; work on it must be enqueued on the
+        stream that is current when the generator is advanced."""
+        n = tensors["tokens"].shape[0]
+        if n == 0:
+            return
+        self._stage(tensors, 0, self.slots[0])
+        for i in range(n):
+            consumer = torch.cuda.current_stream(self.device)
+            if i >= 1:
+                # everything the consumer enqueued for row i-1 precedes this point of its stream
+                self.slots[(i - 1) % self.DEPTH]["released"].record(consumer)
+            if i + 1 < n:
+                self._stage(tensors, i + 1, self.slots[(i + 1) % self.DEPTH])
+            slot = self.slots[i % self.DEPTH]
+            consumer.wait_event(slot["copied"])
+            yield dict(slot["dev"])
+        self.slots[(n - 1) % self.DEPTH]["released"].record(torch.cuda.current_stream(self.device))
 
     def to_device(self, tensors: PackedTensors, row: int) -> PackedTensors:
-        out = {}
-        for key, buf in self.pinned.items():
-            buf.copy_(tensors[key][row:row + 1])
-            out[key] = buf.to(self.device, non_blocking=True)
-        torch.cuda.current_stream(self.device).synchronize()  # the pinned buffers are reused
+        """One row, ready on the current stream (fresh device tensors, no overlap)."""
+        slot = self.slots[0]
+        self._stage(tensors, row, slot)
+        consumer = torch.cuda.current_stream(self.device)
+        consumer.wait_event(slot["copied"])
+        out = {key: t.clone() for key, t in slot["dev"].items()}
+        slot["released"].record(consumer)
         return out

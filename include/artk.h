@@ -253,6 +253,14 @@ int32_t artk_attn_bwd(const void* q, const void* k, const void* v, const void* o
                       int32_t D, const int64_t* strides, float scale, void* dq, void* dk, void* dv,
                       void* workspace, size_t workspace_bytes, artk_stream_t stream);
 
+/* Tuning aid of artk_attn_bwd (no counterpart in the reference).  With grouped-query heads a
+ * key block seen by at most `light_max` (query tile, head) pairs is handled by one work-group
+ * for all heads of its group; busier blocks get one work-group per head and a fixed-order
+ * reduction.  The library picks the threshold by itself (64 for rows long enough to fill the
+ * GPU that way, else 0); this call overrides it for later artk_attn_bwd calls made on the
+ * calling thread, light_max < 0 restores the automatic choice.  Results agree to rounding. */
+int32_t artk_attn_bwd_tuning(int32_t light_max);
+
 /* ------------------------------------------------------------------------- *
  * Optimizer step over the adapter parameters kept in one flat fp32 buffer.
  * Replaces: the per-tensor AdamW step and gradient clipping that HF Trainer runs

@@ -49,7 +49,7 @@ def calculate_logprobs(
     """
     batch, seq_len, _ = hidden_states.shape
     assert seq_len % chunk_size == 0  # train.py:82-84
-    out = torch.empty((batch, seq_len), dtype=hidden_states.dtype)
+    out = torch.empty((batch, seq_len), dtype=hidden_states.dtype, device=hidden_states.device)
     lm_head_t = lm_head_t.to(hidden_states.dtype)
     for i in range(0, seq_len, chunk_size):
         logits = torch.matmul(hidden_states[:, i : i + chunk_size, :], lm_head_t)

@@ -245,14 +245,14 @@ def test_attn_bwd_mixed_light_and_heavy_key_blocks(artk_lib, gpu):
     # both regimes present with the threshold of large rows: first key block heavy, last one light
     assert (S // 64) * Hq > 64 and 2 * Hq <= 64
     results = {}
-    for knob in ("64", "0"):  # the library picks 0 by itself for a row this short
-        os.environ["ARTK_ATTN_LIGHT_MAX"] = knob
+    for knob in (64, 0):  # the library picks 0 by itself for a row this short
+        artk_lib.artk_attn_bwd_tuning(knob)
         try:
             dq, dk, dv = ops.attn_bwd(qd, kd, vd, out, lse, d_out.to(gpu), plan)
         finally:
-            del os.environ["ARTK_ATTN_LIGHT_MAX"]
+            artk_lib.artk_attn_bwd_tuning(-1)
         assert rel_l2(dq.float().cpu(), ref_dq) <= 1e-2
         assert rel_l2(dk.float().cpu(), ref_dk) <= 1e-2
         assert rel_l2(dv.float().cpu(), ref_dv) <= 1e-2
         results[knob] = (dk, dv)
-    assert rel_l2(results["64"][0].float(), results["0"][0].float()) <= 4e-3
+    assert rel_l2(results[64][0].float(), results[0][0].float()) <= 4e-3

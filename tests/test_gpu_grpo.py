@@ -337,3 +337,68 @@ def test_full_size_windows_and_properties(artk_lib, gpu, name):
     assert torch.equal(lp4[(~dead).to(gpu)], lp[(~dead).to(gpu)])
     assert rel_l2(dh4.float(), dh.float()) <= 2e-3
     assert dh4[dead.to(gpu)].abs().max().item() == 0.0
+
+
+def chunk_bounds(T, V):
+    """First positions of the chunks the library forms by itself (chunk_tokens = 0): about 6000
+    positions per chunk, the batch's 256-position tiles spread evenly over the chunks."""
+    cap = max(((1 << 30) - 1) // V // 256 * 256, 256)
+    want = min(cap, 6144)
+    n = -(-T // want)
+    tc = min(-(-(-(-T // n)) // 256) * 256, cap, T)
+    nchunks, tiles = -(-T // tc), -(-T // 256)
+    base, extra = divmod(tiles, nchunks)
+    bounds, t0 = [], 0
+    for c in range(nchunks):
+        bounds.append(t0)
+        t0 += (base + (1 if c < extra else 0)) * 256
+    return bounds
+
+
+@pytest.mark.parametrize("name", ["c3", "c4"])
+def test_full_size_library_chunking_and_independent_loss(artk_lib, gpu, name):
+    """Benchmark configs 3 and 4 with the chunking the library picks by itself (uneven chunks:
+    22 + 21 + 21 tiles at the 7B shape): windows across a chunk boundary, inside the last chunk
+    and at the end of the batch against the CPU oracle; then the WHOLE batch (every logprob, the
+    loss, every d_hidden row) against the oracle's own code evaluated in fp32 by torch on the GPU,
+    which shares nothing with the kernels."""
+    print(f"full size, library chunking {name}", flush=True)
+    case = synthetic.config3() if name == "c3" else synthetic.config4()
+    T, H = case.hidden.shape[1], case.hidden.shape[2]
+    V = case.lm_head.shape[0]
+    args, s, lp, dh, new = run_full_size(case, gpu, 0)
+    count = grpo_oracle.shift_tensor(case.assistant_mask, False).sum().item()
+    assert s[3].item() == count
+    assert torch.equal(lp, new)
+    bounds = chunk_bounds(T, V)
+    assert len(bounds) >= 3 and bounds[1] - bounds[0] != bounds[-1] - bounds[-2]  # uneven chunks
+    starts = (bounds[1] - 48, bounds[-1] - 48, bounds[-1] + 700, T - 96)
+    for start in starts:
+        ref_lp, ref_dh = window_oracle(case, start, 96, count)
+        got_lp = lp[start:start + 95].cpu()
+        got_dh = dh[start:start + 95].float().cpu()
+        assert (got_lp - ref_lp).abs().max().item() <= LP_TOL, start
+        if ref_dh.abs().max().item() == 0.0:
+            assert got_dh.abs().max().item() == 0.0
+        else:
+            assert rel_l2(got_dh, ref_dh) <= GRAD_TOL, start
+    # same batch with even chunks of 4096: forward identical, gradient to rounding
+    s2, lp2, dh2 = ops.grpo_fused(*args, 4096)
+    assert torch.equal(lp2, lp)
+    assert rel_l2(dh2.float(), dh.float()) <= 1e-3
+    del dh2
+    # whole batch against the oracle's code in fp32 on the GPU (rocBLAS fp32 matmul, torch
+    # logsumexp / gather / autograd): an evaluation independent of the kernels at full size
+    g = lambda t: t.to(gpu)
+    ref = grpo_oracle.loss_and_grad(g(case.hidden), g(case.lm_head), g(case.tokens), g(case.logprobs),
+                                    g(case.advantages), g(case.assistant_mask), g(case.weights), chunk_size=1024)
+    assert (lp - ref["logprobs"][0]).abs().max().item() <= LP_TOL
+    assert abs(s[0].item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item())
+    assert abs(s[1].item() - ref["policy_loss"].item()) <= LOSS_TOL * abs(ref["policy_loss"].item())
+    assert rel_l2(dh.float(), ref["d_hidden"][0]) <= GRAD_TOL
+    # row by row, so that a few wrong rows cannot hide in the global norm
+    num = (dh.float() - ref["d_hidden"][0]).norm(dim=1)
+    den = ref["d_hidden"][0].norm(dim=1)
+    live = den > 0
+    assert (num[live] / den[live]).max().item() <= 3e-2
+    assert dh[~live].abs().max().item() == 0.0

@@ -131,6 +131,34 @@ def test_config5_gate_projection_full_size(artk_lib, gpu):
     assert rel_l2(dB.cpu(), dB0) <= TOL
 
 
+def test_config5_down_projection_full_size(artk_lib, gpu):
+    """Benchmark config 5, down projection [2048,768] at full size: 65536 sorted rows of width 768
+    (no gather: the rows are the gated activations, already in expert order), forward and backward."""
+    print("moe config5 down projection", flush=True)
+    T, H, I, E, k = 8192, 2048, 768, 128, 8
+    g = torch.Generator().manual_seed(1005)
+    logits = torch.randn(T, E, generator=g)
+    r, ref = check_routing(logits, k, gpu)
+    h = torch.randn(T * k, I, generator=g).to(torch.bfloat16)
+    W, A, B = make_experts(E, H, I, 8, 2005)
+    up = torch.randn(T * k, H, generator=g).to(torch.bfloat16)
+    y0, dx0, dA0, dB0 = moe_oracle.grouped_lora_grads(h, None, W, A, B, 2.0, ref["offsets"], up)
+    y, xa = ops.moe_lora_grouped_fwd(h.to(gpu), None, W.to(gpu), A.to(gpu), B.to(gpu), 2.0, r)
+    dx, dA, dB = ops.moe_lora_grouped_bwd(up.to(gpu), h.to(gpu), None, ops.transpose_batched(W.to(gpu)),
+                                          A.to(gpu), B.to(gpu), xa, 2.0, r)
+    assert rel_l2(y.cpu().float(), y0) <= TOL
+    assert rel_l2(dx.cpu().float(), dx0) <= TOL
+    assert rel_l2(dA.cpu(), dA0) <= TOL
+    assert rel_l2(dB.cpu(), dB0) <= TOL
+    # per expert as well: a wrong expert boundary would hide in the global norm
+    off = ref["offsets"].tolist()
+    for e in (0, 1, 63, 127):
+        sl = slice(off[e], off[e + 1])
+        assert rel_l2(y[sl].cpu().float(), y0[sl]) <= TOL
+        assert rel_l2(dx[sl].cpu().float(), dx0[sl]) <= TOL
+        assert rel_l2(dA[e].cpu(), dA0[e]) <= TOL and rel_l2(dB[e].cpu(), dB0[e]) <= TOL
+
+
 def test_moe_block_autograd(artk_lib, gpu):
     """The whole block (gate, up, SiLU gating, down, recombination) against torch fp32."""
     torch.manual_seed(0)
