@@ -16,7 +16,7 @@ namespace artk {
 // Work-group shape of each GEMM kernel (see gemm_nt.hpp).
 constexpr int FWD_NI = 2;   // lm_head projection + log-sum-exp epilogue: 8 waves
 constexpr int BWD_NI = 2;   // d_hidden GEMM
-constexpr int GEMM_NI = 2;  // plain GEMM
+constexpr int GEMM_NI = 4;  // plain GEMM: 4 waves, pinned order (+2..4 % over the 8-wave shape)
 
 // ----------------------------------------------------------------------------
 // index helpers
@@ -696,22 +696,15 @@ struct GemmParams {
   int MT, NT, out_f32;
 };
 
-__global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  int mt, nt;
-  tile_coords(id, p.MT, p.NT, mt, nt);
-  TileAcc<GEMM_NI> acc;
-  acc.zero();
-  gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
-               (int)p.K);
+template <int NI>
+__device__ __forceinline__ void gemm_nt_store(const TileAcc<NI>& acc, const GemmParams& p, int mt, int nt) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wm = wave_m<GEMM_NI>(wave), wn = wave_n<GEMM_NI>(wave);
+  const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
   const int half = lane >> 5;
 #pragma unroll
-  for (int ni = 0; ni < GEMM_NI; ++ni) {
-    const int64_t col = (int64_t)nt * TILE + acc_col<GEMM_NI>(wn, ni, lane);
+  for (int ni = 0; ni < NI; ++ni) {
+    const int64_t col = (int64_t)nt * TILE + acc_col<NI>(wn, ni, lane);
     if (col >= p.N) continue;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -732,6 +725,18 @@ __global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams
         }
       }
   }
+}
+
+__global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const int id = xcd_remap(blockIdx.x, gridDim.x);
+  int mt, nt;
+  tile_coords(id, p.MT, p.NT, mt, nt);
+  TileAcc<GEMM_NI> acc;
+  acc.zero();
+  gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
+               (int)p.K);
+  gemm_nt_store<GEMM_NI>(acc, p, mt, nt);
 }
 
 // ----------------------------------------------------------------------------
