@@ -33,6 +33,8 @@ SIGNATURES = {
         _i32,
         [_p, _p, _p, _p, _p, _p, _i32, _i64, _i64, _f32, _f32, _f32, _p, _p, _p, _sz, _p],
     ),
+    "artk_grpo_loss_static": (
+        _i32, [_p, _p, _p, _p, _p, _p, _i32, _i64, _i64, _f32, _f32, _f32, _p, _p, _p]),
     "artk_grpo_fused_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "artk_grpo_fused": (
         _i32,

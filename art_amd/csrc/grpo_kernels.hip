@@ -11,6 +11,8 @@
 
 #include <math.h>
 
+#include <mutex>
+
 namespace artk {
 
 // Work-group shape of each GEMM kernel (see gemm_nt.hpp).
@@ -902,6 +904,42 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   return ARTK_OK;
 }
 
+// ----------------------------------------------------------------------------
+// Scratch of artk_grpo_loss_static: a device array that is part of the code
+// object, so the entry point needs no allocation.  Every GPU the library runs on
+// holds its own copy at its own address; the array's name is only a handle for
+// hipGetSymbolAddress on the host, never a device pointer.
+// ----------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_BYTES =
+    2 * ((size_t)ARTK_GRPO_LOSS_STATIC_MAX_T * sizeof(float) + 256) + 64 * sizeof(int) + 512;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[STATIC_MAX_DEVICES];  // device address of `scratch` per device, once resolved
+static std::mutex g_scratch_mu;
+
+// Device address of `scratch` on the current device (resolved on the first call per device).
+static int32_t static_scratch_base(void** out) {
+  int dev = -1;
+  ARTK_CHECK_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES) {
+    set_error("device ordinal %d outside [0, %d)", dev, STATIC_MAX_DEVICES);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    ARTK_CHECK_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) {
+      set_error("hipGetSymbolAddress returned a null address for the static scratch");
+      return ARTK_ERR_INVALID_ARGUMENT;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return ARTK_OK;
+}
+
 }  // namespace artk
 
 using namespace artk;
@@ -1063,7 +1101,7 @@ size_t artk_grpo_loss_workspace_bytes(int64_t T) {
   return ws.used + 256;
 }
 
-// Body of artk_grpo_loss: the scratch (two f32 [T]
+// Shared body of artk_grpo_loss and artk_grpo_loss_static: the scratch (two f32 [T]
 // arrays of per-token terms and the mask count) is carved out of `ws`.
 static int32_t grpo_loss_run(const float* new_logprob, const float* old_logprob, const float* advantages,
                              const uint8_t* mask, const float* weights, const float* ref_logprob,
@@ -1113,6 +1151,24 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
                        float* scalars, float* coef, void* workspace, size_t workspace_bytes,
                        artk_stream_t stream) {
   Workspace ws(workspace, workspace_bytes);
+  return grpo_loss_run(new_logprob, old_logprob, advantages, mask, weights, ref_logprob, shift, T, S,
+                       clip_lo, clip_hi, beta, scalars, coef, ws, (hipStream_t)stream);
+}
+
+int32_t artk_grpo_loss_static(const float* new_logprob, const float* old_logprob, const float* advantages,
+                              const uint8_t* mask, const float* weights, const float* ref_logprob,
+                              int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi,
+                              float beta, float* scalars, float* coef, artk_stream_t stream) {
+  if (T > ARTK_GRPO_LOSS_STATIC_MAX_T) {
+    set_error("artk_grpo_loss_static handles at most %d positions per call, got %lld (use artk_grpo_loss "
+              "with a caller-provided workspace)",
+              ARTK_GRPO_LOSS_STATIC_MAX_T, (long long)T);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  void* base = nullptr;
+  const int32_t rc = static_scratch_base(&base);
+  if (rc) return rc;
+  Workspace ws(base, STATIC_SCRATCH_BYTES);
   return grpo_loss_run(new_logprob, old_logprob, advantages, mask, weights, ref_logprob, shift, T, S,
                        clip_lo, clip_hi, beta, scalars, coef, ws, (hipStream_t)stream);
 }

@@ -96,6 +96,26 @@ int32_t artk_grpo_loss(const float* new_logprob, const float* old_logprob, const
                        artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * artk_grpo_loss without a workspace argument and without any allocation.
+ * No counterpart in the reference: it exists for callers that cannot allocate
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid the
+ * allocator).  Same arguments, kernels and results as artk_grpo_loss; the
+ * scratch (two f32 [T] arrays and a counter) lives in a device array inside the
+ * library's code object (about 2 MiB per GPU the library runs on, held until
+ * the process ends).  T above ARTK_GRPO_LOSS_STATIC_MAX_T is rejected with
+ * ARTK_ERR_UNSUPPORTED_SHAPE.  The first call on a device looks up the array's
+ * address (hipGetSymbolAddress) and should be made outside a capture.  All calls
+ * on one GPU share the array: calls that overlap on one GPU (different streams
+ * or threads) race; nothing in it has to start at zero (every element a call
+ * reads is written by that call first).
+ * ------------------------------------------------------------------------- */
+#define ARTK_GRPO_LOSS_STATIC_MAX_T 262144
+int32_t artk_grpo_loss_static(const float* new_logprob, const float* old_logprob, const float* advantages,
+                              const uint8_t* mask, const float* weights, const float* ref_logprob,
+                              int32_t shift, int64_t T, int64_t S, float clip_lo, float clip_hi,
+                              float beta, float* scalars, float* coef, artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * A1+A2+A4+A7 fused — loss and d_hidden of one packed batch in one call.
  * Replaces: the body of compute_loss, src/art/local/train.py:76-151, plus the
  *   backward that HF Trainer.training_step triggers on its result.
