@@ -45,7 +45,7 @@ SIGNATURES = {
     "artk_gemm_nt": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _p]),
     "artk_lora_linear_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "artk_lora_linear_fwd": (
-        _i32, [_p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
+        _i32, [_p, _p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
     "artk_lora_linear_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "artk_lora_linear_bwd": (
         _i32, [_p, _p, _p, _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),

@@ -2,8 +2,10 @@
 
 ``LoRALinear`` is the counterpart of the peft ``lora.Linear`` module that the
 reference installs on the attention and MLP projections
-(src/art/local/state.py:86-92; defaults r = 8, alpha = 16, no dropout, no bias:
-src/art/dev/model.py:52-67).  The base weight is frozen; only ``lora_A`` and
+(src/art/local/state.py:86-92; defaults r = 8, alpha = 16, no dropout,
+``bias="none"``: src/art/dev/model.py:52-67).  The base weight is frozen, and so
+is the base layer's own bias when it has one (Qwen2.5's q/k/v projections do;
+peft keeps it and ``bias="none"`` means it is not trained); only ``lora_A`` and
 ``lora_B`` receive gradients."""
 from __future__ import annotations
 
@@ -17,12 +19,12 @@ from . import ops
 
 class _LoRALinearFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, lora_A, lora_B, scale):
+    def forward(ctx, x, weight, lora_A, lora_B, scale, bias=None):
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1]).to(torch.bfloat16).contiguous()
         A = lora_A.detach().to(torch.bfloat16).contiguous()
         B = lora_B.detach().to(torch.bfloat16).contiguous()
-        y, xa = ops.lora_linear_fwd(x2, weight, A, B, scale)
+        y, xa = ops.lora_linear_fwd(x2, weight, A, B, scale, bias)
         ctx.save_for_backward(x2, weight, A, B, xa)
         ctx.scale = scale
         ctx.lead = lead
@@ -35,24 +37,30 @@ class _LoRALinearFn(torch.autograd.Function):
         g2 = g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous()
         dx, dA, dB = ops.lora_linear_bwd(g2, x2, ops.transposed_weight(weight), A, B, xa, ctx.scale)
         a_dtype, b_dtype, x_dtype = ctx.param_dtypes
-        return (dx.view(*ctx.lead, x2.shape[-1]).to(x_dtype), None, dA.to(a_dtype), dB.to(b_dtype), None)
+        return (dx.view(*ctx.lead, x2.shape[-1]).to(x_dtype), None, dA.to(a_dtype), dB.to(b_dtype), None, None)
 
 
-def lora_linear(x, weight, lora_A, lora_B, scale: float):
-    """y = x W^T + scale * (x A^T) B^T with gradients for x, A and B (W frozen)."""
-    return _LoRALinearFn.apply(x, weight, lora_A, lora_B, float(scale))
+def lora_linear(x, weight, lora_A, lora_B, scale: float, bias=None):
+    """y = x W^T + bias + scale * (x A^T) B^T with gradients for x, A and B (W and bias frozen)."""
+    if bias is not None:
+        if bias.requires_grad:
+            raise ValueError("the bias of a LoRA-wrapped linear is frozen (peft bias='none'); got requires_grad=True")
+        bias = bias.detach().to(torch.bfloat16).contiguous()
+    return _LoRALinearFn.apply(x, weight, lora_A, lora_B, float(scale), bias)
 
 
 class LoRALinear(nn.Module):
     """Frozen bf16 linear with a trainable rank-r update; forward(x) -> y."""
 
     def __init__(self, in_features: int, out_features: int, r: int = 8, lora_alpha: int = 16,
-                 device=None, dtype=torch.bfloat16):
+                 device=None, dtype=torch.bfloat16, bias: bool = False):
         super().__init__()
         self.in_features, self.out_features, self.r = in_features, out_features, r
         self.scaling = lora_alpha / r
         self.weight = nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=torch.bfloat16),
                                    requires_grad=False)
+        self.bias = (nn.Parameter(torch.zeros(out_features, device=device, dtype=torch.bfloat16), requires_grad=False)
+                     if bias else None)
         self.lora_A = nn.Parameter(torch.empty(r, in_features, device=device, dtype=dtype))
         self.lora_B = nn.Parameter(torch.zeros(out_features, r, device=device, dtype=dtype))
         self.reset_parameters()
@@ -64,15 +72,16 @@ class LoRALinear(nn.Module):
 
     @classmethod
     def from_linear(cls, linear: nn.Linear, r: int = 8, lora_alpha: int = 16) -> "LoRALinear":
-        if linear.bias is not None:
-            raise ValueError("LoRALinear wraps bias-free projections only")
-        mod = cls(linear.in_features, linear.out_features, r, lora_alpha, device=linear.weight.device)
+        mod = cls(linear.in_features, linear.out_features, r, lora_alpha, device=linear.weight.device,
+                  bias=linear.bias is not None)
         with torch.no_grad():
             mod.weight.copy_(linear.weight.to(torch.bfloat16))
+            if linear.bias is not None:
+                mod.bias.copy_(linear.bias.to(torch.bfloat16))
         return mod
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return lora_linear(x, self.weight, self.lora_A, self.lora_B, self.scaling)
+        return lora_linear(x, self.weight, self.lora_A, self.lora_B, self.scaling, self.bias)
 
 
 class _FusedLoRAFn(torch.autograd.Function):
@@ -81,7 +90,7 @@ class _FusedLoRAFn(torch.autograd.Function):
     sum(r_i) update whose B factor is block-diagonal."""
 
     @staticmethod
-    def forward(ctx, x, weight_cat, scale, outs, ranks, *AB):
+    def forward(ctx, x, weight_cat, bias_cat, scale, outs, ranks, *AB):
         lead = x.shape[:-1]
         n = len(outs)
         As, Bs = AB[:n], AB[n:]
@@ -93,7 +102,7 @@ class _FusedLoRAFn(torch.autograd.Function):
             B_bd[o0:o0 + o, r0:r0 + r] = b.detach().to(torch.bfloat16)
             o0 += o
             r0 += r
-        y, xa = ops.lora_linear_fwd(x2, weight_cat, A_cat, B_bd, scale)
+        y, xa = ops.lora_linear_fwd(x2, weight_cat, A_cat, B_bd, scale, bias_cat)
         ctx.save_for_backward(x2, weight_cat, A_cat, B_bd, xa)
         ctx.meta = (scale, lead, outs, ranks, [a.dtype for a in As], [b.dtype for b in Bs], x.dtype)
         return y.view(*lead, sum(outs))
@@ -111,7 +120,7 @@ class _FusedLoRAFn(torch.autograd.Function):
             dBs.append(dB[o0:o0 + o, r0:r0 + r].to(bd))   # off-diagonal blocks belong to no adapter
             o0 += o
             r0 += r
-        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, None, None, *dAs, *dBs)
+        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, None, None, None, *dAs, *dBs)
 
 
 class FusedLoRALinear(nn.Module):
@@ -133,10 +142,16 @@ class FusedLoRALinear(nn.Module):
         self.scaling = layers[0].scaling
         self.weight = nn.Parameter(torch.cat([l.weight.detach() for l in layers], 0).contiguous(),
                                    requires_grad=False)
+        if any(l.bias is not None for l in layers):   # frozen biases; projections without one add zero
+            parts = [l.bias.detach() if l.bias is not None else
+                     torch.zeros(l.out_features, dtype=torch.bfloat16, device=l.weight.device) for l in layers]
+            self.bias = nn.Parameter(torch.cat(parts).to(torch.bfloat16).contiguous(), requires_grad=False)
+        else:
+            self.bias = None
         self.lora_A = nn.ParameterList([l.lora_A for l in layers])
         self.lora_B = nn.ParameterList([l.lora_B for l in layers])
 
     def forward(self, x: torch.Tensor):
-        y = _FusedLoRAFn.apply(x, self.weight, float(self.scaling), self.outs, self.ranks, *self.lora_A,
-                               *self.lora_B)
+        y = _FusedLoRAFn.apply(x, self.weight, self.bias, float(self.scaling), self.outs, self.ranks,
+                               *self.lora_A, *self.lora_B)
         return torch.split(y, self.outs, dim=-1)

@@ -264,22 +264,25 @@ def grpo_fused_workspace_bytes(T: int, V: int, H: int, chunk_tokens: int = DEFAU
 # -----------------------------------------------------------------------------
 # LoRA linear
 # -----------------------------------------------------------------------------
-def lora_linear_fwd(x, W, A, B, scale: float):
-    """(y bf16 [T,out], xa f32 [T,r]) for x bf16 [T,in], W bf16 [out,in], A bf16 [r,in], B bf16 [out,r]."""
+def lora_linear_fwd(x, W, A, B, scale: float, bias: Optional[torch.Tensor] = None):
+    """(y bf16 [T,out], xa f32 [T,r]) for x bf16 [T,in], W bf16 [out,in], A bf16 [r,in], B bf16 [out,r]
+    and an optional frozen bias bf16 [out] (added in the GEMM epilogue)."""
     T, n_in = x.shape
     n_out, r = B.shape
     _need(x, "x", torch.bfloat16)
     _need(W, "W", torch.bfloat16, (n_out, n_in))
     _need(A, "A", torch.bfloat16, (r, n_in))
     _need(B, "B", torch.bfloat16, (n_out, r))
+    if bias is not None:
+        _need(bias, "bias", torch.bfloat16, (n_out,))
     lib = _lib.load()
     dev = x.device
     y = torch.empty((T, n_out), dtype=torch.bfloat16, device=dev)
     xa = torch.empty((T, r), dtype=torch.float32, device=dev)
     ws = _workspace(lib.artk_lora_linear_fwd_workspace_bytes(T, n_in, n_out, r), dev)
     _lib.check(
-        lib.artk_lora_linear_fwd(x.data_ptr(), W.data_ptr(), A.data_ptr(), B.data_ptr(), scale, T,
-                                 n_in, n_out, r, y.data_ptr(), xa.data_ptr(), ws.data_ptr(),
+        lib.artk_lora_linear_fwd(x.data_ptr(), W.data_ptr(), A.data_ptr(), B.data_ptr(), _ptr(bias), scale,
+                                 T, n_in, n_out, r, y.data_ptr(), xa.data_ptr(), ws.data_ptr(),
                                  ws.numel(), _stream(dev))
     )
     return y, xa

@@ -164,7 +164,10 @@ def base_result(args, metric, unit, value, ms_per_step, workload):
 def bench_lora(args):
     """LoRA linear fwd+bwd over the six projections of one Qwen2.5-3B layer that have
     in = 2048 (q, o: out 2048; k, v: out 256; gate, up: out 11008), T = 8192, r = 8, alpha = 16.
-    One step = forward + backward of all six; value = algorithmic TFLOP/s of the step."""
+    One step = forward + backward of all six.  `value` = algorithmic TFLOP/s of the step when the
+    projections that read the same activations run as one product (q/k/v and gate/up, the way
+    art_amd.lora.FusedLoRALinear runs them: weights concatenated along the output dimension,
+    adapters stacked with a block-diagonal B); `separate` = the same six as six calls."""
     import math
 
     import torch
@@ -174,59 +177,91 @@ def bench_lora(args):
     dev = torch.device("cuda:0")
     T, n_in, r, scale = 8192, 2048, 8, 2.0
     g = torch.Generator().manual_seed(1002)
-    x = torch.randn(T, n_in, generator=g).to(torch.bfloat16).to(dev)
-    shapes = []
+    x_cpu = torch.randn(T, n_in, generator=g).to(torch.bfloat16)
+    x = x_cpu.to(dev)
+    cpu, shapes = {}, {}
     for name, n_out in (("q", 2048), ("o", 2048), ("k", 256), ("v", 256), ("gate", 11008), ("up", 11008)):
-        W = (0.02 * torch.randn(n_out, n_in, generator=g)).to(torch.bfloat16).to(dev)
-        A = ((torch.rand(r, n_in, generator=g) * 2 - 1) / math.sqrt(n_in)).to(torch.bfloat16).to(dev)
-        B = (0.01 * torch.randn(n_out, r, generator=g)).to(torch.bfloat16).to(dev)
-        up = torch.randn(T, n_out, generator=g).to(torch.bfloat16).to(dev)
-        shapes.append((name, n_out, W, ops.transpose(W), A, B, up))
+        W = (0.02 * torch.randn(n_out, n_in, generator=g)).to(torch.bfloat16)
+        A = ((torch.rand(r, n_in, generator=g) * 2 - 1) / math.sqrt(n_in)).to(torch.bfloat16)
+        B = (0.01 * torch.randn(n_out, r, generator=g)).to(torch.bfloat16)
+        up = torch.randn(T, n_out, generator=g).to(torch.bfloat16)
+        cpu[name] = (W, A, B, up)
+        Wd = W.to(dev)
+        shapes[name] = (n_out, Wd, ops.transpose(Wd), A.to(dev), B.to(dev), up.to(dev))
     flops = lambda n_out: 4.0 * T * n_in * n_out + 6.0 * T * r * (n_in + n_out)
+    total = sum(flops(sh[0]) for sh in shapes.values())
 
     def one(sh):
-        _, _, W, Wt, A, B, up = sh
+        _, W, Wt, A, B, up = sh
         y, xa = ops.lora_linear_fwd(x, W, A, B, scale)
-        ops.lora_linear_bwd(up, x, Wt, A, B, xa, scale)
+        return (y,) + ops.lora_linear_bwd(up, x, Wt, A, B, xa, scale)
 
-    def step():
-        for sh in shapes:
+    def fuse(names):
+        parts = [shapes[n] for n in names]
+        W = torch.cat([p[1] for p in parts], 0).contiguous()
+        A = torch.cat([p[3] for p in parts], 0).contiguous()
+        B = torch.zeros(W.shape[0], A.shape[0], dtype=torch.bfloat16, device=dev)
+        o0 = r0 = 0
+        for p in parts:
+            B[o0:o0 + p[0], r0:r0 + r] = p[4]
+            o0, r0 = o0 + p[0], r0 + r
+        up = torch.cat([p[5] for p in parts], 1).contiguous()
+        return (W.shape[0], W, ops.transpose(W), A, B, up)
+
+    fused = {"qkv": fuse(("q", "k", "v")), "o": shapes["o"], "gate_up": fuse(("gate", "up"))}
+
+    def step_separate():
+        for sh in shapes.values():
+            one(sh)
+
+    def step_fused():
+        for sh in fused.values():
             one(sh)
 
     per_shape = {}
-    for sh in shapes[::2]:
+    for name in ("q", "k", "gate"):
+        sh = shapes[name]
         dt = timed(lambda: one(sh), args.steps, args.warmup)
-        per_shape[f"out={sh[1]}"] = {"us_fwd_bwd": dt * 1e6, "tflops": flops(sh[1]) / dt / 1e12,
-                                     "frac": flops(sh[1]) / dt / 1e12 / PEAK_BF16_TFLOPS}
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+        per_shape[f"out={sh[0]}"] = {"us_fwd_bwd": dt * 1e6, "tflops": flops(sh[0]) / dt / 1e12,
+                                     "frac": flops(sh[0]) / dt / 1e12 / PEAK_BF16_TFLOPS}
+    per_fused = {}
+    for name, members in (("qkv", ("q", "k", "v")), ("gate_up", ("gate", "up"))):
+        sh = fused[name]
+        fl = sum(flops(shapes[m][0]) for m in members)
+        dt = timed(lambda: one(sh), args.steps, args.warmup)
+        per_fused[name] = {"out": sh[0], "rank": len(members) * r, "us_fwd_bwd": dt * 1e6,
+                           "tflops": fl / dt / 1e12, "frac": fl / dt / 1e12 / PEAK_BF16_TFLOPS}
+    dt_sep = timed(step_separate, args.steps, args.warmup)
+    dt = timed(step_fused, args.steps, args.warmup)
+    # dominant kernel, from a separate burst with the library's HIP-event brackets on
     ops.profile_enable(True)
-    t0 = time.perf_counter()
     for _ in range(args.steps):
-        one(shapes[4])
+        one(fused["gate_up"])
     torch.cuda.synchronize()
     gemm_ms, gemm_n = ops.profile_collect(ops.PROF_LORA_GEMM)
     ops.profile_enable(False)
-    dt = timed(step, args.steps, 0)
-    total = sum(flops(sh[1]) for sh in shapes)
     res = base_result(args, "LoRA linear fwd+bwd TFLOP/s (Qwen2.5-3B shapes)", "TFLOP/s", total / dt / 1e12,
                       dt * 1e3, "C2-lora-qwen2.5-3b")
-    res["config"].update({"tokens": T, "in": n_in, "rank": r, "projections": "q,o,k,v,gate,up"})
+    res["config"].update({"tokens": T, "in": n_in, "rank": r, "projections": "q,o,k,v,gate,up",
+                          "path": "q/k/v and gate/up as one product each (FusedLoRALinear), o alone"})
     res["frac_of_bf16_peak"] = total / dt / 1e12 / PEAK_BF16_TFLOPS
-    res["shapes"] = per_shape
+    res["fused_products"] = per_fused
+    res["separate"] = {"value": total / dt_sep / 1e12, "unit": "TFLOP/s", "ms_per_step": dt_sep * 1e3,
+                       "frac_of_bf16_peak": total / dt_sep / 1e12 / PEAK_BF16_TFLOPS, "shapes": per_shape,
+                       "note": "six separate calls; per shape: one projection fwd+bwd"}
     launch_ms = gemm_ms / max(gemm_n, 1)
-    ach = 2.0 * T * n_in * 11008 / (launch_ms * 1e-3) / 1e12
-    res["roofline"] = {"kernel": "lora_gemm_kernel (gate/up, fwd and dx launches)", "bound": "mfma",
-                       "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms}
+    ach = 2.0 * T * n_in * 22016 / (launch_ms * 1e-3) / 1e12
+    res["roofline"] = {"kernel": "lora_gemm_kernel (fused gate/up: mean of the y and dx launches)",
+                       "bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms,
+                       "flop_per_launch": 2.0 * T * n_in * 22016}
     if not args.no_secondary:
         # The LoRA linear the way peft evaluates it, in stock torch ops on the same GPU:
         # base(x) + scale * lora_B(lora_A(x)), autograd for dx, dA, dB (W frozen).
         import torch.nn.functional as F
 
         def torch_step():
-            for _, _, W, _, A, B, up in shapes:
+            for _, W, _, A, B, up in shapes.values():
                 xg = x.detach().requires_grad_(True)
                 Ag, Bg = A.detach().requires_grad_(True), B.detach().requires_grad_(True)
                 y = F.linear(xg, W) + scale * F.linear(F.linear(xg, Ag), Bg)
@@ -240,13 +275,46 @@ def bench_lora(args):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import lora_oracle
 
-        _, n_out, W, _, A, B, up = shapes[0]
+        # CPU oracle (fp32) of q, k and v: the timing sample, and the parity reference of this run for
+        # the separate calls (y, dx, dA, dB of q and k) and for the fused q/k/v product (dx is the sum)
+        ref, times = {}, []
+        for rep in range(4):           # 1 warm-up + 3 runs
+            t0 = time.perf_counter()
+            for name in ("q", "k", "v"):
+                W, A, B, up = cpu[name]
+                ref[name] = lora_oracle.lora_linear_grads(x_cpu, W, A, B, scale, up)
+            if rep:
+                times.append(time.perf_counter() - t0)
+        cdt = sorted(times)[1]
         t0 = time.perf_counter()
-        lora_oracle.lora_linear_grads(x.cpu(), W.cpu(), A.cpu(), B.cpu(), scale, up.cpu())
-        cdt = time.perf_counter() - t0
-        res["cpu_baseline"] = {"value": flops(n_out) / cdt / 1e12, "unit": "TFLOP/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"q projection (out=2048) fwd+bwd, fp32 torch-CPU oracle, 1 run of {cdt:.1f} s"}
+        for name in ("q", "k", "v"):
+            W, A, B, up = cpu[name]
+            lora_oracle.lora_linear_grads(x_cpu, W, A, B, scale, up, dtype=torch.bfloat16)
+        cdt16 = time.perf_counter() - t0
+        fl = sum(flops(shapes[n][0]) for n in ("q", "k", "v"))
+        res["cpu_baseline"] = {"value": fl / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                               "kind": "port",
+                               "sample": f"q, k and v projections fwd+bwd, fp32 torch-CPU oracle, 1 warm-up + 3 runs, "
+                                         f"median {cdt:.2f} s",
+                               "bf16": {"value": fl / cdt16 / 1e12, "unit": "TFLOP/s",
+                                        "sample": f"same in bf16, one run of {cdt16:.2f} s"}}
+        rel = lambda a, b: ((a.double().cpu() - b.double()).norm() / b.double().norm()).item()
+        parity = {}
+        for name in ("q", "k"):
+            got = one(shapes[name])
+            parity[name] = dict(zip(("y", "dx", "dA", "dB"), (rel(a, b) for a, b in zip(got, ref[name]))))
+        y, dx, dA, dB = one(fused["qkv"])
+        o0 = r0 = 0
+        fq = {"dx": rel(dx, ref["q"][1] + ref["k"][1] + ref["v"][1])}
+        for name in ("q", "k", "v"):
+            n_out = shapes[name][0]
+            fq[f"y_{name}"] = rel(y[:, o0:o0 + n_out], ref[name][0])
+            fq[f"dA_{name}"] = rel(dA[r0:r0 + r], ref[name][2])
+            fq[f"dB_{name}"] = rel(dB[o0:o0 + n_out, r0:r0 + r], ref[name][3])
+            o0, r0 = o0 + n_out, r0 + r
+        parity["fused_qkv"] = fq
+        parity["tolerance_rel_l2"] = 1e-2
+        res["parity_same_run"] = parity
     return res
 
 

@@ -161,19 +161,24 @@ int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t
  *   the seven projection modules (src/art/local/state.py:86-92,
  *   src/art/dev/model.py:52-67; arithmetic in the third-party package).
  *   x bf16 [T,in], W bf16 [out,in] (frozen), A bf16 [r,in], B bf16 [out,r]
+ *   bias bf16 [out] or NULL: the frozen bias of the wrapped linear (Qwen2.5 has one on
+ *        q/k/v; peft keeps the base layer's bias), added in the GEMM epilogue: y += bias
  *   y bf16 [T,out] out, xa f32 [T,r] out (x A^T, kept for the backward)
  * Requires in % 64 == 0, out % 64 == 0, r % 8 == 0, r <= 64.
  * ------------------------------------------------------------------------- */
 size_t artk_lora_linear_fwd_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r);
-int32_t artk_lora_linear_fwd(const void* x, const void* W, const void* A, const void* B, float scale,
-                             int64_t T, int64_t in, int64_t out, int32_t r, void* y, float* xa,
+int32_t artk_lora_linear_fwd(const void* x, const void* W, const void* A, const void* B, const void* bias,
+                             float scale, int64_t T, int64_t in, int64_t out, int32_t r, void* y, float* xa,
                              void* workspace, size_t workspace_bytes, artk_stream_t stream);
 
 /* Backward of the above for upstream gradient g bf16 [T,out]:
  *   dx bf16 [T,in] = g W + scale (g B) A
  *   dA f32 [r,in]  = scale (g B)^T x        dB f32 [out,r] = scale g^T (x A^T)
  * Replaces: autograd of peft's lora.Linear (W frozen, so no dW).
- *   W_t bf16 [in,out]: transposed copy of W (artk_transpose_bf16); xa from the forward. */
+ *   W_t bf16 [in,out]: transposed copy of W (artk_transpose_bf16); xa from the forward.
+ * g is read from HBM once for g B and dB together (and once more by the dx GEMM), x once
+ * for dA; the sums over column chunks / row slabs are taken in a fixed order.
+ * xa, dA, dB 16-byte aligned. */
 size_t artk_lora_linear_bwd_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r);
 int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, const void* A,
                              const void* B, const float* xa, float scale, int64_t T, int64_t in,

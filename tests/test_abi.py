@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound(artk_lib):
     for n in names:
         assert hasattr(artk_lib, n), f"{n} declared in artk.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
-    assert artk_lib.artk_abi_version() == 2
+    assert artk_lib.artk_abi_version() == 3
 
 
 def test_argument_errors_have_codes_and_messages(artk_lib):
@@ -45,7 +45,7 @@ def test_argument_errors_have_codes_and_messages(artk_lib):
     assert rc == _lib.ERR_WORKSPACE_TOO_SMALL
     rc = artk_lib.artk_grpo_loss(p, p, p, p, p, None, 0, 64, 64, 1.5, 0.5, 0.0, p, p, p, 4096, None)
     assert rc == _lib.ERR_INVALID_ARGUMENT  # clip_lo > clip_hi
-    rc = artk_lib.artk_lora_linear_fwd(p, p, p, p, 2.0, 64, 64, 64, 5, p, p, p, 4096, None)  # rank 5
+    rc = artk_lib.artk_lora_linear_fwd(p, p, p, p, None, 2.0, 64, 64, 64, 5, p, p, p, 4096, None)  # rank 5
     assert rc == _lib.ERR_UNSUPPORTED_SHAPE
     # gathered MoE rows further than 2 GiB from x
     rc = artk_lib.artk_moe_lora_grouped_fwd(p, p, p, p, p, 2.0, p, p, p, 1 << 20, 4096, 64, 8, 8, p, p, p, 4096, None)

@@ -140,3 +140,44 @@ def test_fused_projections_match_separate(artk_lib, gpu):
     assert rel(x2.grad.float(), x1.grad.float()) <= 1e-2
     for l, (dA, dB) in zip(layers, ref):
         assert rel(l.lora_A.grad, dA) <= 1e-2 and rel(l.lora_B.grad, dB) <= 1e-2
+
+
+@pytest.mark.parametrize("n_out,r", [(2048, 8), (256, 8), (320, 48)])
+def test_lora_bias_and_ranks(artk_lib, gpu, n_out, r):
+    """Qwen2.5's q/k/v projections carry a (frozen) bias: y = x W^T + bias + s (x A^T) B^T at the
+    config-2 q and k/v shapes, and a rank above 32 on a ragged shape (two e tiles in the
+    one-pass skinny products).  The bias adds nothing to dx, dA, dB."""
+    print(f"lora bias out={n_out} r={r}", flush=True)
+    T, n_in = (8192, 2048) if r == 8 else (1100, 448)
+    x, W, A, B, up = make(T, n_in, n_out, r, 77 + n_out)
+    bias = (0.5 * torch.randn(n_out, generator=torch.Generator().manual_seed(n_out))).to(torch.bfloat16)
+    scale = 16 / r
+    y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, scale, up)
+    y0 = y0 + bias.float()
+    xd, Wd, Ad, Bd, upd = (t.to(gpu) for t in (x, W, A, B, up))
+    y, xa = ops.lora_linear_fwd(xd, Wd, Ad, Bd, scale, bias.to(gpu))
+    dx, dA, dB = ops.lora_linear_bwd(upd, xd, ops.transpose(Wd), Ad, Bd, xa, scale)
+    assert rel_l2(y.cpu().float(), y0) <= TOL
+    assert rel_l2(dx.cpu().float(), dx0) <= TOL
+    assert rel_l2(dA.cpu(), dA0) <= TOL
+    assert rel_l2(dB.cpu(), dB0) <= TOL
+    # bit-reproducible run to run (fixed summation orders)
+    dx2, dA2, dB2 = ops.lora_linear_bwd(upd, xd, ops.transpose(Wd), Ad, Bd, xa, scale)
+    assert torch.equal(dA, dA2) and torch.equal(dB, dB2) and torch.equal(dx, dx2)
+
+
+def test_lora_module_with_bias_from_linear(artk_lib, gpu):
+    """LoRALinear.from_linear keeps the base layer's bias (as peft does) and leaves it frozen."""
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(256, 192, bias=True, device=gpu, dtype=torch.bfloat16)
+    mod = LoRALinear.from_linear(lin, r=8, lora_alpha=16)
+    assert mod.bias is not None and not mod.bias.requires_grad
+    with torch.no_grad():
+        mod.lora_B.normal_(std=0.02)
+    x = torch.randn(300, 256, device=gpu, dtype=torch.bfloat16, requires_grad=True)
+    y = mod(x)
+    y.backward(torch.ones_like(y))
+    want = (x.detach().float() @ lin.weight.float().t() + lin.bias.float()
+            + mod.scaling * (x.detach().float() @ mod.lora_A.float().t()) @ mod.lora_B.float().t())
+    assert rel_l2(y.detach().float().cpu(), want.cpu()) <= TOL
+    assert mod.bias.grad is None and mod.lora_A.grad is not None
