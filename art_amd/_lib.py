@@ -79,6 +79,24 @@ SIGNATURES = {
     "artk_stream_copy": (_i32, [_p, _p, _i64, _p]),
 }
 
+
+
+class Nf4Struct(C.Structure):
+    """artk_nf4_t of include/artk.h."""
+    _fields_ = [("packed", _p), ("absmax", _p), ("absmax_q", _p), ("code2", _p), ("absmax2", _p),
+                ("offset", _f32), ("blocksize", _i32)]
+
+
+SIGNATURES.update({
+    "artk_nf4_dequant_t": (_i32, [_p, _p, _p, _p, _p, _f32, _i64, _i64, _i32, _p, _p]),
+    "artk_lora_linear_fwd_nf4_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "artk_lora_linear_fwd_nf4": (
+        _i32, [_p, C.POINTER(Nf4Struct), _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
+    "artk_lora_linear_bwd_nf4_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "artk_lora_linear_bwd_nf4": (
+        _i32, [_p, _p, C.POINTER(Nf4Struct), _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),
+})
+
 _lib = None
 
 

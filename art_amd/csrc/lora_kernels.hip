@@ -825,4 +825,71 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
   return ARTK_OK;
 }
 
+// ---- the same linear with the frozen weight kept as NF4 codes -------------------------------
+// The bf16 weight exists only inside the call: it is dequantised into the workspace (forward:
+// [out,in]; backward: [in,out], written transposed straight from the codes), consumed by the
+// GEMM and forgotten, so neither a bf16 copy nor a transposed copy of W stays resident.
+static int32_t check_nf4_weight(const artk_nf4_t* W, int64_t in) {
+  ARTK_CHECK_ARG(W != nullptr && W->packed != nullptr, "null NF4 weight");
+  ARTK_CHECK_ARG(W->blocksize >= 32 && in % W->blocksize == 0,
+                 "the input size must be a multiple of the quantisation block size");
+  return ARTK_OK;
+}
+
+size_t artk_lora_linear_fwd_nf4_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r) {
+  Workspace ws(nullptr, 0);
+  ws.take<uint16_t>((size_t)out * in);
+  ws.take<char>(artk_lora_linear_fwd_workspace_bytes(T, in, out, r));
+  return ws.used + 256;
+}
+
+int32_t artk_lora_linear_fwd_nf4(const void* x, const artk_nf4_t* W, const void* A, const void* B,
+                                 const void* bias, float scale, int64_t T, int64_t in, int64_t out, int32_t r,
+                                 void* y, float* xa, void* workspace, size_t workspace_bytes,
+                                 artk_stream_t stream) {
+  int32_t rc = check_lora(T, in, out, r);
+  if (rc) return rc;
+  if ((rc = check_nf4_weight(W, in))) return rc;
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* Wd = ws.take<uint16_t>((size_t)out * in);
+  const size_t inner = artk_lora_linear_fwd_workspace_bytes(T, in, out, r);
+  char* rest = ws.take<char>(inner);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  if ((rc = artk_nf4_dequant(W->packed, W->absmax, W->absmax_q, W->code2, W->absmax2, W->offset, out * in,
+                             W->blocksize, Wd, stream)))
+    return rc;
+  return artk_lora_linear_fwd(x, Wd, A, B, bias, scale, T, in, out, r, y, xa, rest, inner, stream);
+}
+
+size_t artk_lora_linear_bwd_nf4_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r) {
+  Workspace ws(nullptr, 0);
+  ws.take<uint16_t>((size_t)out * in);
+  ws.take<char>(artk_lora_linear_bwd_workspace_bytes(T, in, out, r));
+  return ws.used + 256;
+}
+
+int32_t artk_lora_linear_bwd_nf4(const void* g, const void* x, const artk_nf4_t* W, const void* A,
+                                 const void* B, const float* xa, float scale, int64_t T, int64_t in,
+                                 int64_t out, int32_t r, void* dx, float* dA, float* dB, void* workspace,
+                                 size_t workspace_bytes, artk_stream_t stream) {
+  int32_t rc = check_lora(T, in, out, r);
+  if (rc) return rc;
+  if ((rc = check_nf4_weight(W, in))) return rc;
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* Wt = ws.take<uint16_t>((size_t)out * in);
+  const size_t inner = artk_lora_linear_bwd_workspace_bytes(T, in, out, r);
+  char* rest = ws.take<char>(inner);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  if ((rc = artk_nf4_dequant_t(W->packed, W->absmax, W->absmax_q, W->code2, W->absmax2, W->offset, out, in,
+                               W->blocksize, Wt, stream)))
+    return rc;
+  return artk_lora_linear_bwd(g, x, Wt, A, B, xa, scale, T, in, out, r, dx, dA, dB, rest, inner, stream);
+}
+
 }  // extern "C"

@@ -40,12 +40,40 @@ class _LoRALinearFn(torch.autograd.Function):
         return (dx.view(*ctx.lead, x2.shape[-1]).to(x_dtype), None, dA.to(a_dtype), dB.to(b_dtype), None, None)
 
 
+class _LoRALinearNF4Fn(torch.autograd.Function):
+    """The same linear with the frozen weight kept as NF4 codes (art_amd.quant.NF4Weight)."""
+
+    @staticmethod
+    def forward(ctx, x, w_nf4, lora_A, lora_B, scale, bias=None):
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1]).to(torch.bfloat16).contiguous()
+        A = lora_A.detach().to(torch.bfloat16).contiguous()
+        B = lora_B.detach().to(torch.bfloat16).contiguous()
+        y, xa = ops.lora_linear_fwd_nf4(x2, w_nf4, A, B, scale, bias)
+        ctx.save_for_backward(x2, A, B, xa)
+        ctx.w_nf4 = w_nf4
+        ctx.scale = scale
+        ctx.lead = lead
+        ctx.param_dtypes = (lora_A.dtype, lora_B.dtype, x.dtype)
+        return y.view(*lead, w_nf4.shape[0])
+
+    @staticmethod
+    def backward(ctx, g):
+        x2, A, B, xa = ctx.saved_tensors
+        g2 = g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous()
+        dx, dA, dB = ops.lora_linear_bwd_nf4(g2, x2, ctx.w_nf4, A, B, xa, ctx.scale)
+        a_dtype, b_dtype, x_dtype = ctx.param_dtypes
+        return (dx.view(*ctx.lead, x2.shape[-1]).to(x_dtype), None, dA.to(a_dtype), dB.to(b_dtype), None, None)
+
+
 def lora_linear(x, weight, lora_A, lora_B, scale: float, bias=None):
     """y = x W^T + bias + scale * (x A^T) B^T with gradients for x, A and B (W and bias frozen)."""
     if bias is not None:
         if bias.requires_grad:
             raise ValueError("the bias of a LoRA-wrapped linear is frozen (peft bias='none'); got requires_grad=True")
         bias = bias.detach().to(torch.bfloat16).contiguous()
+    if not isinstance(weight, torch.Tensor):   # an NF4Weight
+        return _LoRALinearNF4Fn.apply(x, weight, lora_A, lora_B, float(scale), bias)
     return _LoRALinearFn.apply(x, weight, lora_A, lora_B, float(scale), bias)
 
 
@@ -80,8 +108,29 @@ class LoRALinear(nn.Module):
                 mod.bias.copy_(linear.bias.to(torch.bfloat16))
         return mod
 
+    @classmethod
+    def from_nf4(cls, w_nf4, r: int = 8, lora_alpha: int = 16, bias=None) -> "LoRALinear":
+        """Wrap a frozen weight that stays in its 4-bit storage form (art_amd.quant.NF4Weight): the
+        module then holds no 16-bit copy of it, as with `load_in_4bit=True` in the reference
+        (src/art/dev/model.py:29)."""
+        n_out, n_in = w_nf4.shape
+        dev = w_nf4.packed.device
+        mod = cls.__new__(cls)
+        nn.Module.__init__(mod)
+        mod.in_features, mod.out_features, mod.r = n_in, n_out, r
+        mod.scaling = lora_alpha / r
+        mod.weight = None
+        mod.weight_nf4 = w_nf4
+        mod.bias = (nn.Parameter(bias.detach().to(torch.bfloat16).to(dev), requires_grad=False)
+                    if bias is not None else None)
+        mod.lora_A = nn.Parameter(torch.empty(r, n_in, device=dev, dtype=torch.bfloat16))
+        mod.lora_B = nn.Parameter(torch.zeros(n_out, r, device=dev, dtype=torch.bfloat16))
+        nn.init.kaiming_uniform_(mod.lora_A, a=math.sqrt(5))
+        return mod
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return lora_linear(x, self.weight, self.lora_A, self.lora_B, self.scaling, self.bias)
+        weight = self.weight if self.weight is not None else self.weight_nf4
+        return lora_linear(x, weight, self.lora_A, self.lora_B, self.scaling, self.bias)
 
 
 class _FusedLoRAFn(torch.autograd.Function):

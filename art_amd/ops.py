@@ -508,6 +508,82 @@ def nf4_dequant(packed, absmax=None, absmax_q=None, code2=None, absmax2=None, of
     return out
 
 
+def nf4_dequant_t(packed, rows: int, cols: int, absmax=None, absmax_q=None, code2=None, absmax2=None,
+                  offset: float = 0.0, blocksize: int = 64) -> torch.Tensor:
+    """bf16 [cols, rows]: the [rows, cols] weight behind the NF4 codes, written transposed."""
+    _need(packed, "packed", torch.uint8, (rows * cols // 2,))
+    out = torch.empty((cols, rows), dtype=torch.bfloat16, device=packed.device)
+    _lib.check(_lib.load().artk_nf4_dequant_t(packed.data_ptr(), _ptr(absmax), _ptr(absmax_q), _ptr(code2),
+                                              _ptr(absmax2), offset, rows, cols, blocksize, out.data_ptr(),
+                                              _stream(packed.device)))
+    return out
+
+
+def _nf4_struct(w) -> "_lib.Nf4Struct":
+    """artk_nf4_t for an art_amd.quant.NF4Weight (the tensors stay owned by `w`)."""
+    n = w.shape[0] * w.shape[1]
+    _need(w.packed, "packed", torch.uint8, (n // 2,))
+    if w.absmax is not None:
+        _need(w.absmax, "absmax", torch.float32, (n // w.blocksize,))
+    else:
+        _need(w.absmax_q, "absmax_q", torch.uint8, (n // w.blocksize,))
+        _need(w.code2, "code2", torch.float32, (256,))
+        _need(w.absmax2, "absmax2", torch.float32)
+    return _lib.Nf4Struct(w.packed.data_ptr(), _ptr(w.absmax), _ptr(w.absmax_q), _ptr(w.code2), _ptr(w.absmax2),
+                          float(w.offset), int(w.blocksize))
+
+
+def lora_linear_fwd_nf4(x, w_nf4, A, B, scale: float, bias: Optional[torch.Tensor] = None):
+    """lora_linear_fwd with the frozen weight given as NF4 codes (art_amd.quant.NF4Weight); the
+    bf16 weight lives in the call's workspace only."""
+    import ctypes as C
+
+    T, n_in = x.shape
+    n_out, r = B.shape
+    if tuple(w_nf4.shape) != (n_out, n_in):
+        raise ValueError(f"NF4 weight has shape {tuple(w_nf4.shape)}, expected {(n_out, n_in)}")
+    _need(x, "x", torch.bfloat16)
+    _need(A, "A", torch.bfloat16, (r, n_in))
+    _need(B, "B", torch.bfloat16, (n_out, r))
+    if bias is not None:
+        _need(bias, "bias", torch.bfloat16, (n_out,))
+    lib = _lib.load()
+    dev = x.device
+    y = torch.empty((T, n_out), dtype=torch.bfloat16, device=dev)
+    xa = torch.empty((T, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_lora_linear_fwd_nf4_workspace_bytes(T, n_in, n_out, r), dev)
+    st = _nf4_struct(w_nf4)
+    _lib.check(lib.artk_lora_linear_fwd_nf4(x.data_ptr(), C.byref(st), A.data_ptr(), B.data_ptr(), _ptr(bias),
+                                            scale, T, n_in, n_out, r, y.data_ptr(), xa.data_ptr(),
+                                            ws.data_ptr(), ws.numel(), _stream(dev)))
+    return y, xa
+
+
+def lora_linear_bwd_nf4(g, x, w_nf4, A, B, xa, scale: float):
+    """lora_linear_bwd with the frozen weight given as NF4 codes; no transposed copy is kept."""
+    import ctypes as C
+
+    T, n_in = x.shape
+    n_out, r = B.shape
+    _need(g, "g", torch.bfloat16, (T, n_out))
+    _need(x, "x", torch.bfloat16)
+    _need(A, "A", torch.bfloat16, (r, n_in))
+    _need(B, "B", torch.bfloat16, (n_out, r))
+    _need(xa, "xa", torch.float32, (T, r))
+    lib = _lib.load()
+    dev = x.device
+    dx = torch.empty((T, n_in), dtype=torch.bfloat16, device=dev)
+    dA = torch.empty((r, n_in), dtype=torch.float32, device=dev)
+    dB = torch.empty((n_out, r), dtype=torch.float32, device=dev)
+    ws = _workspace(lib.artk_lora_linear_bwd_nf4_workspace_bytes(T, n_in, n_out, r), dev)
+    st = _nf4_struct(w_nf4)
+    _lib.check(lib.artk_lora_linear_bwd_nf4(g.data_ptr(), x.data_ptr(), C.byref(st), A.data_ptr(), B.data_ptr(),
+                                            xa.data_ptr(), scale, T, n_in, n_out, r, dx.data_ptr(),
+                                            dA.data_ptr(), dB.data_ptr(), ws.data_ptr(), ws.numel(),
+                                            _stream(dev)))
+    return dx, dA, dB
+
+
 # -----------------------------------------------------------------------------
 # Optimizer
 # -----------------------------------------------------------------------------

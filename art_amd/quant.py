@@ -2,8 +2,12 @@
 
 With `load_in_4bit=True` (src/art/dev/model.py:29) the reference's frozen linear
 weights are stored as NF4 codes by bitsandbytes and dequantised in front of every
-matmul.  `NF4Weight` holds that storage form on the GPU and produces the bf16
-weight (and its transposed copy for the backward) that `art_amd.lora` consumes.
+matmul.  `NF4Weight` holds that storage form on the GPU.  `art_amd.lora.LoRALinear`
+takes it as its frozen weight (`LoRALinear.from_nf4`): the bf16 values then exist only
+inside each forward / backward call, in the call's workspace, so neither a bf16 copy
+nor a transposed copy stays resident (0.56 bytes per weight element instead of 4).
+`dequantize()` / `dequantize_transposed()` give resident bf16 tensors for callers that
+prefer to pay the memory (no dequantisation per call: about 3 % of a projection's time).
 """
 from __future__ import annotations
 
@@ -47,5 +51,11 @@ class NF4Weight:
         return flat.view(self.shape)
 
     def dequantize_transposed(self) -> torch.Tensor:
-        """bf16 [in, out], the operand of the input-gradient GEMM."""
-        return ops.transpose(self.dequantize())
+        """bf16 [in, out], the operand of the input-gradient GEMM, written transposed straight from the codes."""
+        return ops.nf4_dequant_t(self.packed, self.shape[0], self.shape[1], self.absmax, self.absmax_q,
+                                 self.code2, self.absmax2, self.offset, self.blocksize)
+
+    def nbytes(self) -> int:
+        """Bytes of device memory the storage form occupies."""
+        return sum(t.numel() * t.element_size() for t in
+                   (self.packed, self.absmax, self.absmax_q, self.code2, self.absmax2) if t is not None)

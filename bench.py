@@ -679,6 +679,36 @@ def bench_nf4(args):
     gbs = 2.5625 * n / dt / 1e9
     res["roofline"] = {"kernel": "nf4_dequant_kernel", "bound": "hbm", "achieved": gbs, "peak": 8000.0,
                        "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None}
+    # The two ways to run a LoRA projection on a 4-bit base weight (gate projection of config 2:
+    # 8192 tokens, 2048 -> 11008, rank 8), forward + backward: bf16 weight and transposed copy
+    # resident (dequantised once), or the 4-bit form only and the 16-bit weight inside each call.
+    from art_amd.quant import NF4Weight
+
+    T, n_in, n_out, r = 8192, 2048, 11008, 8
+    q = NF4Weight(torch.randint(0, 256, (n_out * n_in // 2,), generator=g, dtype=torch.uint8).to(dev),
+                  (n_out, n_in), absmax=(0.05 * torch.rand(n_out * n_in // 64, generator=g)).to(dev))
+    x = torch.randn(T, n_in, generator=g).to(torch.bfloat16).to(dev)
+    A = (0.02 * torch.randn(r, n_in, generator=g)).to(torch.bfloat16).to(dev)
+    B = (0.01 * torch.randn(n_out, r, generator=g)).to(torch.bfloat16).to(dev)
+    up = torch.randn(T, n_out, generator=g).to(torch.bfloat16).to(dev)
+    Wd, Wt = q.dequantize(), q.dequantize_transposed()
+
+    def resident():
+        y, xa = ops.lora_linear_fwd(x, Wd, A, B, 2.0)
+        ops.lora_linear_bwd(up, x, Wt, A, B, xa, 2.0)
+
+    def transient():
+        y, xa = ops.lora_linear_fwd_nf4(x, q, A, B, 2.0)
+        ops.lora_linear_bwd_nf4(up, x, q, A, B, xa, 2.0)
+
+    t_res = timed(resident, args.steps, args.warmup)
+    t_tr = timed(transient, args.steps, args.warmup)
+    res["lora_on_nf4_base"] = {
+        "shape": {"tokens": T, "in": n_in, "out": n_out, "rank": r},
+        "resident_bf16": {"us_fwd_bwd": t_res * 1e6, "weight_bytes_resident": 4 * n_out * n_in + q.nbytes()},
+        "nf4_only": {"us_fwd_bwd": t_tr * 1e6, "weight_bytes_resident": q.nbytes(),
+                     "transient_workspace_bytes": 2 * n_out * n_in},
+        "time_ratio": t_tr / t_res}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import quant_oracle

@@ -322,6 +322,41 @@ int32_t artk_adamw_step(float* params, const float* grads, float* exp_avg, float
 int32_t artk_nf4_dequant(const void* packed, const float* absmax, const void* absmax_q,
                          const float* code2, const float* absmax2, float offset, int64_t n,
                          int32_t blocksize, void* out_bf16, artk_stream_t stream);
+/* The same values written transposed: the codes are a [rows, cols] matrix (blocks run along a
+ * row), out_bf16 is [cols, rows].  rows, cols multiples of 8. */
+int32_t artk_nf4_dequant_t(const void* packed, const float* absmax, const void* absmax_q,
+                           const float* code2, const float* absmax2, float offset, int64_t rows,
+                           int64_t cols, int32_t blocksize, void* out_bf16, artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
+ * LoRA linear whose frozen weight stays in its NF4 storage form.
+ * Replaces: the 4-bit base linear + peft lora.Linear pair of a model loaded with
+ *   `load_in_4bit=True` (src/art/dev/model.py:29): bitsandbytes dequantises the weight in
+ *   front of every matmul and keeps no 16-bit copy.
+ * Same arguments and results as artk_lora_linear_fwd / _bwd, bit for bit, for the bf16 values
+ * that artk_nf4_dequant gives; the 16-bit weight exists only inside the call, in the
+ * workspace (forward: [out,in]; backward: [in,out], dequantised transposed), so no bf16
+ * copy and no transposed copy of W stay resident between calls.
+ * ------------------------------------------------------------------------- */
+typedef struct artk_nf4 {
+  const void* packed;    /* u8 [out*in/2] */
+  const float* absmax;   /* f32 [out*in/blocksize], or NULL with the double-quantised form: */
+  const void* absmax_q;  /* u8 [out*in/blocksize] */
+  const float* code2;    /* f32 [256] */
+  const float* absmax2;  /* f32 [ceil(out*in/blocksize/256)] */
+  float offset;
+  int32_t blocksize;     /* power of two >= 32 that divides `in` */
+} artk_nf4_t;
+size_t artk_lora_linear_fwd_nf4_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r);
+int32_t artk_lora_linear_fwd_nf4(const void* x, const artk_nf4_t* W, const void* A, const void* B,
+                                 const void* bias, float scale, int64_t T, int64_t in, int64_t out, int32_t r,
+                                 void* y, float* xa, void* workspace, size_t workspace_bytes,
+                                 artk_stream_t stream);
+size_t artk_lora_linear_bwd_nf4_workspace_bytes(int64_t T, int64_t in, int64_t out, int32_t r);
+int32_t artk_lora_linear_bwd_nf4(const void* g, const void* x, const artk_nf4_t* W, const void* A,
+                                 const void* B, const float* xa, float scale, int64_t T, int64_t in,
+                                 int64_t out, int32_t r, void* dx, float* dA, float* dB, void* workspace,
+                                 size_t workspace_bytes, artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
