@@ -88,6 +88,8 @@ class Nf4Struct(C.Structure):
 
 
 SIGNATURES.update({
+    "artk_adamw8bit_step": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _f32, _i32,
+                                   _p, _f32, _p]),
     "artk_nf4_dequant_t": (_i32, [_p, _p, _p, _p, _p, _f32, _i64, _i64, _i32, _p, _p]),
     "artk_lora_linear_fwd_nf4_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "artk_lora_linear_fwd_nf4": (

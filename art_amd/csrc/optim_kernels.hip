@@ -110,6 +110,84 @@ __global__ __launch_bounds__(256) void adamw_kernel(AdamWParams a) {
   }
 }
 
+// ----------------------------------------------------------------------------
+// AdamW with 8-bit block-wise moments (the storage form of `paged_adamw_8bit`).
+// Each moment is one byte per element: an index into a 256-entry code book of
+// values in [-1, 1] (exp_avg) or [0, 1] (exp_avg_sq), times one fp32 absolute
+// maximum per block of 256 elements.  One work-group = one block: dequantise,
+// update in fp32, new block maxima, requantise to the nearest code.
+// ----------------------------------------------------------------------------
+struct AdamW8Params {
+  float* p;
+  const float* g;
+  uint8_t* c1;
+  uint8_t* c2;
+  float* absmax1;
+  float* absmax2;
+  const float* qmap1;
+  const float* qmap2;
+  uint16_t* p_bf16;
+  const float* grad_sumsq;
+  int64_t n;
+  float lr, beta1, beta2, eps, weight_decay, max_grad_norm;
+  float step_size;   // -lr * sqrt(1 - beta2^t) / (1 - beta1^t)
+  float eps_scaled;  // sqrt(1 - beta2^t) * eps
+};
+
+// Index of the entry of the ascending code book nearest to x (ties to the lower index).
+__device__ __forceinline__ int nearest_code(const float* map, float x) {
+  int lo = 0, hi = 255;  // invariant: map[lo] <= x (or lo == 0), map[hi] >= x (or hi == 255)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (map[mid] <= x) lo = mid; else hi = mid;
+  }
+  return (x - map[lo] <= map[hi] - x) ? lo : hi;
+}
+
+__global__ __launch_bounds__(256) void adamw8bit_kernel(AdamW8Params a) {
+  __shared__ float map1[256], map2[256];
+  __shared__ float red[2][4];
+  map1[threadIdx.x] = a.qmap1[threadIdx.x];
+  map2[threadIdx.x] = a.qmap2[threadIdx.x];
+  float clip = 1.f;
+  if (a.grad_sumsq != nullptr) {
+    const float c = a.max_grad_norm / (sqrtf(a.grad_sumsq[0]) + 1e-6f);
+    clip = c < 1.f ? c : 1.f;
+  }
+  __syncthreads();
+  const int64_t b = blockIdx.x;
+  const int64_t i = b * 256 + threadIdx.x;
+  const bool in = i < a.n;
+  float m = 0.f, v = 0.f, g = 0.f, pv = 0.f;
+  if (in) {
+    g = a.g[i] * clip;
+    pv = a.p[i];
+    m = map1[a.c1[i]] * a.absmax1[b];
+    v = map2[a.c2[i]] * a.absmax2[b];
+    m = m * a.beta1 + (1.f - a.beta1) * g;
+    v = v * a.beta2 + (1.f - a.beta2) * g * g;
+  }
+  float mx1 = wave_max(fabsf(m)), mx2 = wave_max(fabsf(v));
+  if ((threadIdx.x & 63) == 0) {
+    red[0][threadIdx.x >> 6] = mx1;
+    red[1][threadIdx.x >> 6] = mx2;
+  }
+  __syncthreads();
+  mx1 = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+  mx2 = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
+  if (threadIdx.x == 0) {
+    a.absmax1[b] = mx1;
+    a.absmax2[b] = mx2;
+  }
+  if (!in) return;
+  pv = pv + a.step_size * (m / (sqrtf(v) + a.eps_scaled));
+  if (a.weight_decay > 0.f) pv = pv * (1.f - a.lr * a.weight_decay);
+  a.p[i] = pv;
+  if (a.p_bf16) a.p_bf16[i] = f32_to_bf16(pv);
+  a.c1[i] = (uint8_t)nearest_code(map1, mx1 > 0.f ? m / mx1 : 0.f);
+  a.c2[i] = (uint8_t)nearest_code(map2, mx2 > 0.f ? v / mx2 : 0.f);
+}
+
 }  // namespace artk
 
 using namespace artk;
@@ -166,6 +244,42 @@ int32_t artk_adamw_step(float* params, const float* grads, float* exp_avg, float
   a.inv_bc2_sqrt = (float)(1.0 / sqrt(bc2));
   const int64_t n4 = (n + 3) / 4;
   adamw_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, (hipStream_t)stream>>>(a);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_adamw8bit_step(float* params, const float* grads, void* state1, void* state2, float* absmax1,
+                            float* absmax2, const float* qmap1, const float* qmap2, void* params_bf16,
+                            int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
+                            int32_t step, const float* grad_sumsq, float max_grad_norm,
+                            artk_stream_t stream) {
+  ARTK_CHECK_ARG(params && grads && state1 && state2 && absmax1 && absmax2 && qmap1 && qmap2,
+                 "null pointer argument");
+  ARTK_CHECK_ARG(n > 0 && step >= 1, "n must be positive and step >= 1");
+  ARTK_CHECK_ARG(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f, "betas must be in [0, 1)");
+  AdamW8Params a;
+  a.p = params;
+  a.g = grads;
+  a.c1 = (uint8_t*)state1;
+  a.c2 = (uint8_t*)state2;
+  a.absmax1 = absmax1;
+  a.absmax2 = absmax2;
+  a.qmap1 = qmap1;
+  a.qmap2 = qmap2;
+  a.p_bf16 = (uint16_t*)params_bf16;
+  a.grad_sumsq = grad_sumsq;
+  a.n = n;
+  a.lr = lr;
+  a.beta1 = beta1;
+  a.beta2 = beta2;
+  a.eps = eps;
+  a.weight_decay = weight_decay;
+  a.max_grad_norm = max_grad_norm;
+  const double c1 = 1.0 - pow((double)beta1, (double)step);
+  const double c2 = sqrt(1.0 - pow((double)beta2, (double)step));
+  a.step_size = (float)(-(double)lr * c2 / c1);
+  a.eps_scaled = (float)(c2 * (double)eps);
+  adamw8bit_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(a);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

@@ -613,6 +613,27 @@ def adamw_step(p, g, m, v, p_bf16, lr, beta1, beta2, eps, weight_decay, step, gr
                                            _ptr(grad_sumsq), max_grad_norm, _stream(p.device)))
 
 
+def adamw8bit_step(p, g, state1, state2, absmax1, absmax2, qmap1, qmap2, p_bf16, lr, beta1, beta2, eps,
+                   weight_decay, step, grad_sumsq=None, max_grad_norm=0.0) -> None:
+    """In-place AdamW with 8-bit block-wise moments (see artk_adamw8bit_step)."""
+    n = p.numel()
+    nb = (n + 255) // 256
+    _need(p, "p", torch.float32)
+    _need(g, "g", torch.float32, (n,))
+    _need(state1, "state1", torch.uint8, (n,))
+    _need(state2, "state2", torch.uint8, (n,))
+    _need(absmax1, "absmax1", torch.float32, (nb,))
+    _need(absmax2, "absmax2", torch.float32, (nb,))
+    _need(qmap1, "qmap1", torch.float32, (256,))
+    _need(qmap2, "qmap2", torch.float32, (256,))
+    if p_bf16 is not None:
+        _need(p_bf16, "p_bf16", torch.bfloat16)
+    _lib.check(_lib.load().artk_adamw8bit_step(
+        p.data_ptr(), g.data_ptr(), state1.data_ptr(), state2.data_ptr(), absmax1.data_ptr(), absmax2.data_ptr(),
+        qmap1.data_ptr(), qmap2.data_ptr(), _ptr(p_bf16), n, lr, beta1, beta2, eps, weight_decay, step,
+        _ptr(grad_sumsq), max_grad_norm, _stream(p.device)))
+
+
 # -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------

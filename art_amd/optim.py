@@ -1,4 +1,4 @@
-"""Flat storage and fused AdamW for the adapter parameters.
+"""Flat storage and fused AdamW for the adapter parameters (fp32 or 8-bit block-wise moments).
 
 The reference lets HF Trainer step `paged_adamw_8bit` over ~400 small LoRA
 tensors and clip their global gradient norm at 0.1 (src/art/dev/model.py:69-85).
@@ -80,3 +80,76 @@ class FusedAdamW:
                        self.betas[1], self.eps, self.weight_decay, self.steps,
                        sumsq if clip else None, self.max_grad_norm if clip else 0.0)
         return sumsq
+
+
+def dynamic_code_book(signed: bool, max_exponent_bits: int = 7, total_bits: int = 8) -> torch.Tensor:
+    """The 256-entry "dynamic" code book of the 8-bit block-wise optimizers (Dettmers et al.,
+    "8-bit Optimizers via Block-wise Quantization", 2022, section 2.2 / appendix: a sign bit,
+    a run of exponent bits that selects a power of ten, and a linear fraction with the
+    remaining bits), ascending, in [-1, 1] (signed: exp_avg) or [0, 1] (unsigned: exp_avg_sq).
+    Restated from the published construction; bitsandbytes itself is not available here, so
+    the book is an explicit input of the kernel and a checkpoint's own book can be passed instead."""
+    data = []
+    non_sign_bits = total_bits - 1
+    additional_items = 2 ** (non_sign_bits - max_exponent_bits) - 1
+    for i in range(max_exponent_bits):
+        if signed:
+            fraction_items = int(2 ** (i + non_sign_bits - max_exponent_bits) + 1)
+        else:
+            fraction_items = int(2 ** (i + non_sign_bits - max_exponent_bits + 1) + 1)
+        boundaries = torch.linspace(0.1, 1, fraction_items, dtype=torch.float64)
+        means = (boundaries[:-1] + boundaries[1:]) / 2.0
+        scale = 10.0 ** (-(max_exponent_bits - 1) + i)
+        data += (scale * means).tolist()
+        if signed:
+            data += (-scale * means).tolist()
+    if additional_items > 0:
+        boundaries = torch.linspace(0.1, 1, additional_items + 1, dtype=torch.float64)
+        means = (boundaries[:-1] + boundaries[1:]) / 2.0
+        scale = 10.0 ** (-(max_exponent_bits - 1) + max_exponent_bits - 1)
+        data += (scale * means).tolist()
+        if signed:
+            data += (-scale * means).tolist()
+    data += [0.0, 1.0]
+    data += [0.0] * (2 ** total_bits - len(data))
+    return torch.tensor(sorted(data), dtype=torch.float32)
+
+
+class FusedAdamW8bit:
+    """FusedAdamW with the moments kept the way the reference's `paged_adamw_8bit` keeps them
+    (src/art/dev/model.py:75): one byte per element and moment plus one fp32 maximum per block of
+    256 elements, 2 bytes of optimizer state per parameter instead of 8."""
+
+    def __init__(self, flat: FlatParams, lr: float = 5e-6, betas=(0.9, 0.99), eps: float = 1e-8,
+                 weight_decay: float = 0.1, max_grad_norm: float = 0.1):
+        self.flat = flat
+        self.lr, self.betas, self.eps = lr, betas, eps
+        self.weight_decay, self.max_grad_norm = weight_decay, max_grad_norm
+        dev = flat.master.device
+        n, nb = flat.numel, (flat.numel + 255) // 256
+        self.state1 = torch.zeros(n, dtype=torch.uint8, device=dev)
+        self.state2 = torch.zeros(n, dtype=torch.uint8, device=dev)
+        self.absmax1 = torch.zeros(nb, dtype=torch.float32, device=dev)
+        self.absmax2 = torch.zeros(nb, dtype=torch.float32, device=dev)
+        self.qmap1 = dynamic_code_book(True).to(dev)
+        self.qmap2 = dynamic_code_book(False).to(dev)
+        self.steps = 0
+
+    def step(self) -> torch.Tensor:
+        """One update; returns the squared gradient norm before clipping (device scalar)."""
+        self.steps += 1
+        f = self.flat
+        sumsq = ops.sumsq(f.grad)
+        clip = self.max_grad_norm is not None and self.max_grad_norm > 0
+        ops.adamw8bit_step(f.master, f.grad, self.state1, self.state2, self.absmax1, self.absmax2, self.qmap1,
+                           self.qmap2, f.shadow, self.lr, self.betas[0], self.betas[1], self.eps,
+                           self.weight_decay, self.steps, sumsq if clip else None,
+                           self.max_grad_norm if clip else 0.0)
+        return sumsq
+
+    def exp_avg(self) -> torch.Tensor:
+        """The first moment, dequantised (for inspection and tests)."""
+        return self.qmap1[self.state1.long()] * self.absmax1.repeat_interleave(256)[: self.flat.numel]
+
+    def exp_avg_sq(self) -> torch.Tensor:
+        return self.qmap2[self.state2.long()] * self.absmax2.repeat_interleave(256)[: self.flat.numel]

@@ -644,6 +644,15 @@ def bench_optim(args):
     gbs = 34.0 * n / dt / 1e9
     res["roofline"] = {"kernel": "sumsq_partial_kernel + adamw_kernel", "bound": "hbm", "achieved": gbs,
                        "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None}
+    # the same step with the moments in the 8-bit block-wise form of `paged_adamw_8bit`:
+    # 4 B for the norm + 10 B read + 8 B written per parameter, 2 B of state instead of 8
+    from art_amd.optim import FusedAdamW8bit
+
+    opt8 = FusedAdamW8bit(flat)
+    dt8 = timed(opt8.step, args.steps, args.warmup)
+    res["moments_8bit"] = {"value": n / dt8, "unit": "params/s", "ms_per_step": dt8 * 1e3,
+                           "gb_per_s": 22.0 * n / dt8 / 1e9, "state_bytes_per_param": 2 + 8 / 256,
+                           "state_bytes_per_param_f32": 8}
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import optim_oracle

@@ -307,6 +307,22 @@ int32_t artk_adamw_step(float* params, const float* grads, float* exp_avg, float
                         float weight_decay, int32_t step, const float* grad_sumsq, float max_grad_norm,
                         artk_stream_t stream);
 
+/* The same step with the moments in the storage form of `paged_adamw_8bit`
+ * (src/art/dev/model.py:75; the arithmetic is bitsandbytes' block-wise 8-bit optimizer, not in
+ * the reference tree): one byte per element and moment, an index into a 256-entry ascending
+ * code book (qmap1 for exp_avg, values in [-1,1]; qmap2 for exp_avg_sq, values in [0,1]),
+ * times one f32 maximum per block of 256 elements (absmax1 / absmax2, f32 [ceil(n/256)],
+ * zero before the first step).  Per block: dequantise, g' as above,
+ *   m = beta1 m + (1 - beta1) g';  v = beta2 v + (1 - beta2) g'^2;
+ *   p = (p - lr sqrt(1 - beta2^t) / (1 - beta1^t) * m / (sqrt(v) + sqrt(1 - beta2^t) eps)) (1 - lr weight_decay);
+ * new block maxima of |m| and v, each moment stored as the nearest code of m / max (ties to
+ * the lower code).  10 bytes of state and gradient traffic per parameter less than the f32 form. */
+int32_t artk_adamw8bit_step(float* params, const float* grads, void* state1, void* state2, float* absmax1,
+                            float* absmax2, const float* qmap1, const float* qmap2, void* params_bf16,
+                            int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
+                            int32_t step, const float* grad_sumsq, float max_grad_norm,
+                            artk_stream_t stream);
+
 /* ------------------------------------------------------------------------- *
  * NF4 base weight -> bf16.
  * Replaces: the dequantisation that bitsandbytes performs in front of every
