@@ -13,6 +13,7 @@
 #include "common.hpp"
 #include "gemm_nt.hpp"
 #include "lora_common.hpp"
+#include "skinny_stats.hpp"
 
 #include <math.h>
 
@@ -613,14 +614,26 @@ int32_t artk_moe_lora_grouped_fwd(const void* x, const int32_t* gather, const vo
                          out, in, E, r, RP, st);
 }
 
+// Scratch of the grouped backward, carved in the same order by the size query and the call.
+struct MoeBwdScratch {
+  uint16_t *Bt, *At, *gb16;
+  float *gb, *rowp, *dummy;
+};
+static void carve_moe_bwd(Workspace& ws, int64_t n_rows, int64_t in, int64_t out, int E, int r, MoeBwdScratch& c) {
+  const int RP = round16(r);
+  c.Bt = ws.take<uint16_t>((size_t)E * r * out);  // [E,r,out]
+  c.At = ws.take<uint16_t>((size_t)E * in * r);   // [E,in,r]
+  c.gb = ws.take<float>((size_t)n_rows * r);
+  c.gb16 = ws.take<uint16_t>((size_t)n_rows * RP);
+  c.rowp = ws.take<float>((size_t)stats_grouped_chunks(out, r) * n_rows * r);
+  c.dummy = ws.take<float>(1024);
+}
+
 size_t artk_moe_lora_grouped_bwd_workspace_bytes(int64_t n_rows, int64_t in, int64_t out, int32_t E,
                                                  int32_t r) {
-  const int RP = round16(r);
   Workspace ws(nullptr, 0);
-  ws.take<uint16_t>((size_t)E * r * out);
-  ws.take<uint16_t>((size_t)E * in * r);
-  ws.take<float>((size_t)n_rows * r);
-  ws.take<uint16_t>((size_t)n_rows * RP);
+  MoeBwdScratch c;
+  carve_moe_bwd(ws, n_rows, in, out, E, r, c);
   return ws.used + 256;
 }
 
@@ -635,28 +648,43 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
   ARTK_CHECK_ARG(g && x && W_t && A && B && xa && expert_offsets && tile_prefix && blk_prefix && dx &&
                      dA && dB,
                  "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(dx),
+  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(dx) && aligned16(xa) &&
+                     aligned16(dA) && aligned16(dB),
                  "pointers must be 16-byte aligned");
+  if (n_rows * (in > out ? in : out) * 2 >= (1ll << 31)) {
+    set_error("n_rows * max(in, out) * 2 bytes (%lld) must stay below 2 GiB (31-bit row offsets)",
+              (long long)(n_rows * (in > out ? in : out) * 2));
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
-  uint16_t* Bt = ws.take<uint16_t>((size_t)E * r * out);  // [E,r,out]
-  uint16_t* At = ws.take<uint16_t>((size_t)E * in * r);   // [E,in,r]
-  float* gb = ws.take<float>((size_t)n_rows * r);
-  uint16_t* gb16 = ws.take<uint16_t>((size_t)n_rows * RP);
+  MoeBwdScratch c;
+  carve_moe_bwd(ws, n_rows, in, out, E, r, c);
   if (!ws.ok()) {
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
   hipStream_t st = (hipStream_t)stream;
-  if ((rc = launch_small_transpose2(B, Bt, E, out, r, A, At, E, r, in, st))) return rc;
-  if ((rc = launch_moe_rowdot(g, nullptr, Bt, expert_offsets, blk_prefix, n_rows, E, out, r, RP, scale,
-                              gb, gb16, st)))
+  if ((rc = launch_small_transpose2(B, c.Bt, E, out, r, A, c.At, E, r, in, st))) return rc;
+  // one pass over g: g B_e per row (partials over column chunks) and dB_e = s g^T (x A_e^T) per expert
+  if ((rc = launch_stats_grouped(g, n_rows, nullptr, n_rows, out, c.Bt, xa, r, E, expert_offsets, c.rowp, dB,
+                                 scale, 0, c.dummy, st)))
     return rc;
-  if ((rc = launch_moe_gemm(W_t, g, nullptr, At, gb16, dx, expert_offsets, tile_prefix, n_rows, in, out,
+  {
+    StatsReduceJob ja{c.rowp, stats_grouped_chunks(out, r), n_rows, 1.f, c.gb, 0, c.gb16, RP, scale};
+    StatsReduceJob jb{nullptr, 0, 0, 0.f, nullptr, 0, nullptr, 0, 0.f};
+    if ((rc = launch_stats_reduce(ja, jb, r, st))) return rc;
+  }
+  if ((rc = launch_moe_gemm(W_t, g, nullptr, c.At, c.gb16, dx, expert_offsets, tile_prefix, n_rows, in, out,
                             E, r, RP, st)))
     return rc;
-  if ((rc = launch_moe_coldot(x, gather, gb, expert_offsets, E, in, r, scale, 1, dA, st))) return rc;
-  return launch_moe_coldot(g, nullptr, xa, expert_offsets, E, out, r, scale, 0, dB, st);
+  // one pass over x: dA_e [r,in] = s (g B_e)^T x.  (With a row gather the last tile of a row may
+  // reach past the row: only taken when the rows are whole tiles wide, so nothing is read
+  // beyond the last row of x, whose count this call does not know.)
+  if (gather == nullptr || in % ST_TILE == 0)
+    return launch_stats_grouped(x, gather ? (int64_t)0x3fffffff / in : n_rows, gather, n_rows, in, nullptr, c.gb,
+                                r, E, expert_offsets, nullptr, dA, scale, 1, c.dummy, st);
+  return launch_moe_coldot(x, gather, c.gb, expert_offsets, E, in, r, scale, 1, dA, st);
 }
 
 int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_t R, int64_t C,
