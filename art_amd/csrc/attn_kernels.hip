@@ -268,14 +268,26 @@ __device__ __forceinline__ bf16x8 tr_frag(const char* tile, const TrLane& t, int
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// attn_smem_note: the kernels below track the completion of their LDS DMA by hand (wait_vmcnt
+// before the barrier that publishes a stage).  Two things would make the compiler drain every
+// outstanding DMA instead, serialising the ring: a second LDS variable in the kernel (it then
+// puts s_waitcnt vmcnt(0) in front of LDS reads that follow a DMA issue), and __syncthreads(),
+// whose fence waits for all memory operations; hence one LDS array per kernel, carved by
+// hand, and barrier_lds_only() inside the loops.
+// Makes the compiler finish the load of v here (it waits for a value where an instruction first
+// uses it).  Left alone it would put the wait for a prologue load at the first use inside the main
+// loop, where the same s_waitcnt vmcnt(..) then also waits for the DMA ring on every iteration.
+template <class V>
+__device__ __forceinline__ void pin_loaded(V& v) {
+  asm volatile("" : "+v"(v));
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t attn_rsrc(const void* p) {
-  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
-}
+__device__ __forceinline__ dma_rsrc_t attn_rsrc(const void* p) { return dma_make_rsrc(p, 0x7fffffffu); }
 
 // ----------------------------------------------------------------------------
 // Forward
@@ -308,9 +320,9 @@ struct AttnKvStage {
 // DMA of key block kb into one stage: this wave's share of the K and V tiles,
 // plus the 64 key codes (every wave writes the same 256 bytes).
 template <int D>
-__device__ __forceinline__ void attn_issue_kv(char* st, int kb, __amdgpu_buffer_rsrc_t rsrc_k,
-                                              __amdgpu_buffer_rsrc_t rsrc_v,
-                                              __amdgpu_buffer_rsrc_t rsrc_c,
+__device__ __forceinline__ void attn_issue_kv(char* st, int kb, dma_rsrc_t rsrc_k,
+                                              dma_rsrc_t rsrc_v,
+                                              dma_rsrc_t rsrc_c,
                                               const int* voff_k,
                                               const int* voff_v, int64_t k_ss,
                                               int64_t v_ss, int wave, int lane) {
@@ -319,22 +331,20 @@ __device__ __forceinline__ void attn_issue_kv(char* st, int kb, __amdgpu_buffer_
   const int k0 = kb * ATT_BN;
 #pragma unroll
   for (int i = 0; i < T::N8; ++i)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_ptr_t)(st + (wave * T::N8 + i) * 1024), 16,
-                                             voff_k[i], (int)(k0 * k_ss * 2), 0, 0);
+    dma_load16(rsrc_k, voff_k[i], (int)(k0 * k_ss * 2), lds_addr_of(st + (wave * T::N8 + i) * 1024));
 #pragma unroll
   for (int i = 0; i < T::N8; ++i)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, (lds_ptr_t)(st + G::V_OFF + (wave * T::N8 + i) * 1024),
-                                             16, voff_v[i], (int)(k0 * v_ss * 2), 0, 0);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_c, (lds_ptr_t)(st + G::CODE_OFF), 4, lane * 4, k0 * 4, 0,
-                                           0);
+    dma_load16(rsrc_v, voff_v[i], (int)(k0 * v_ss * 2), lds_addr_of(st + G::V_OFF + (wave * T::N8 + i) * 1024));
+  dma_load4(rsrc_c, lane * 4, k0 * 4, lds_addr_of(st + G::CODE_OFF));
 }
 
 template <int D>
 __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
   using T = AttnTile<D>;
   using G = AttnKvStage<D>;
-  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE];
-  __shared__ uint32_t s_list[ATT_MAX_KB];
+  // one LDS object for the stages and the tile list (see attn_smem_note)
+  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE + ATT_MAX_KB * 4];
+  uint32_t* const s_list = (uint32_t*)(smem + ATT_STAGES * G::STAGE);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const TrLane tr(lane);
@@ -353,11 +363,11 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
 #pragma unroll
     for (int s = 0; s < D / 16; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
   }
-  const int gi = p.gc[q], pi = p.pc[q];
+  int gi = p.gc[q], pi = p.pc[q];
 
-  const __amdgpu_buffer_rsrc_t rsrc_k = attn_rsrc(p.K + (int64_t)hkv * p.k_hs);
-  const __amdgpu_buffer_rsrc_t rsrc_v = attn_rsrc(p.V + (int64_t)hkv * p.v_hs);
-  const __amdgpu_buffer_rsrc_t rsrc_c = attn_rsrc(p.gc);
+  const dma_rsrc_t rsrc_k = attn_rsrc(p.K + (int64_t)hkv * p.k_hs);
+  const dma_rsrc_t rsrc_v = attn_rsrc(p.V + (int64_t)hkv * p.v_hs);
+  const dma_rsrc_t rsrc_c = attn_rsrc(p.gc);
   int voff_k[T::N8], voff_v[T::N8];
 #pragma unroll
   for (int i = 0; i < T::N8; ++i) {
@@ -377,6 +387,10 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
     for (int j = 0; j < 16; ++j) o[dt][j] = 0.f;
   float m_run = -1e30f, l_run = 0.f;
 
+#pragma unroll
+  for (int s = 0; s < D / 16; ++s) pin_loaded(qf[s]);
+  pin_loaded(gi);
+  pin_loaded(pi);
   if (cnt > 0) ATTN_ISSUE(0, 0);
   if (cnt > 1) ATTN_ISSUE(1, 1);
   int stage = 0;
@@ -385,7 +399,7 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
       wait_vmcnt<G::N_PER>();
     else
       wait_vmcnt<0>();
-    __syncthreads();
+    barrier_lds_only();
     if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int kb = entry & 0x3fff;
@@ -558,8 +572,9 @@ template <int D>
 __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
   using T = AttnTile<D>;
   using G = AttnKvStage<D>;
-  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE];
-  __shared__ uint32_t s_list[ATT_MAX_KB];
+  // one LDS object for the stages and the tile list (see attn_smem_note)
+  __shared__ __attribute__((aligned(1024))) char smem[ATT_STAGES * G::STAGE + ATT_MAX_KB * 4];
+  uint32_t* const s_list = (uint32_t*)(smem + ATT_STAGES * G::STAGE);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const TrLane tr(lane);
@@ -580,13 +595,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
       dof[s] = *(const bf16x8*)(gp + 16 * s);
     }
   }
-  const int gi = p.gc[q], pi = p.pc[q];
-  const float nlse2 = -p.lse2[(int64_t)hq * p.S + q];
-  const float delta = p.delta[(int64_t)hq * p.S + q];
+  int gi = p.gc[q], pi = p.pc[q];
+  float nlse2 = -p.lse2[(int64_t)hq * p.S + q];
+  float delta = p.delta[(int64_t)hq * p.S + q];
 
-  const __amdgpu_buffer_rsrc_t rsrc_k = attn_rsrc(p.K + (int64_t)hkv * p.k_hs);
-  const __amdgpu_buffer_rsrc_t rsrc_v = attn_rsrc(p.V + (int64_t)hkv * p.v_hs);
-  const __amdgpu_buffer_rsrc_t rsrc_c = attn_rsrc(p.gc);
+  const dma_rsrc_t rsrc_k = attn_rsrc(p.K + (int64_t)hkv * p.k_hs);
+  const dma_rsrc_t rsrc_v = attn_rsrc(p.V + (int64_t)hkv * p.v_hs);
+  const dma_rsrc_t rsrc_c = attn_rsrc(p.gc);
   int voff_k[T::N8], voff_v[T::N8];
 #pragma unroll
   for (int i = 0; i < T::N8; ++i) {
@@ -605,6 +620,15 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) dq[dt][j] = 0.f;
 
+#pragma unroll
+  for (int s = 0; s < D / 16; ++s) {
+    pin_loaded(qf[s]);
+    pin_loaded(dof[s]);
+  }
+  pin_loaded(gi);
+  pin_loaded(pi);
+  pin_loaded(nlse2);
+  pin_loaded(delta);
   if (cnt > 0) ATTN_ISSUE(0, 0);
   if (cnt > 1) ATTN_ISSUE(1, 1);
   int stage = 0;
@@ -613,7 +637,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_kernel(AttnBwdParams p) {
       wait_vmcnt<G::N_PER>();
     else
       wait_vmcnt<0>();
-    __syncthreads();
+    barrier_lds_only();
     if (it + 2 < cnt) ATTN_ISSUE(it + 2, stage >= 1 ? stage - 1 : ATT_STAGES - 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[it]);
     const int kb = entry & 0x3fff;
@@ -702,9 +726,9 @@ struct AttnQStage {
 // one of the four per-query arrays (wave & 3 = 0: lse2, 1: delta, 2: group codes,
 // 3: parent codes; the upper four waves write the same bytes again).
 template <int D>
-__device__ __forceinline__ void attn_issue_q(char* st, int hq, int q0, __amdgpu_buffer_rsrc_t rsrc_q,
-                                             __amdgpu_buffer_rsrc_t rsrc_do,
-                                             __amdgpu_buffer_rsrc_t rsrc_row, const int* voff_q,
+__device__ __forceinline__ void attn_issue_q(char* st, int hq, int q0, dma_rsrc_t rsrc_q,
+                                             dma_rsrc_t rsrc_do,
+                                             dma_rsrc_t rsrc_row, const int* voff_q,
                                              const int* voff_do, const AttnBwdParams& p, int wave,
                                              int lane) {
   using T = AttnTile<D>;
@@ -713,20 +737,17 @@ __device__ __forceinline__ void attn_issue_q(char* st, int hq, int q0, __amdgpu_
   const int so_do = (int)((q0 * p.do_ss + hq * p.do_hs) * 2);
 #pragma unroll
   for (int i = 0; i < T::N8; ++i) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_q, (lds_ptr_t)(st + (wave * T::N8 + i) * 1024), 16,
-                                             voff_q[i], so_q, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_do, (lds_ptr_t)(st + G::DO_OFF + (wave * T::N8 + i) * 1024),
-                                             16, voff_do[i], so_do, 0, 0);
+    dma_load16(rsrc_q, voff_q[i], so_q, lds_addr_of(st + (wave * T::N8 + i) * 1024));
+    dma_load16(rsrc_do, voff_do[i], so_do, lds_addr_of(st + G::DO_OFF + (wave * T::N8 + i) * 1024));
   }
   const int arr = wave & 3;
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row, (lds_ptr_t)(st + G::ROW_OFF + arr * 256), 4, lane * 4,
-                                           (int)(((arr < 2 ? (int64_t)hq * p.S : 0) + q0) * 4), 0, 0);
+  dma_load4(rsrc_row, lane * 4, (int)(((arr < 2 ? (int64_t)hq * p.S : 0) + q0) * 4), lds_addr_of(st + G::ROW_OFF + arr * 256));
 }
 
 // The block's K and V rows (128 each = two 64-row tiles per operand).
 template <int D>
-__device__ __forceinline__ void attn_issue_kv_block(char* dst, int key0, __amdgpu_buffer_rsrc_t rsrc_k,
-                                                    __amdgpu_buffer_rsrc_t rsrc_v, const int* voff_k,
+__device__ __forceinline__ void attn_issue_kv_block(char* dst, int key0, dma_rsrc_t rsrc_k,
+                                                    dma_rsrc_t rsrc_v, const int* voff_k,
                                                     const int* voff_v, int64_t k_ss, int64_t v_ss,
                                                     int wave) {
   using T = AttnTile<D>;
@@ -734,12 +755,8 @@ __device__ __forceinline__ void attn_issue_kv_block(char* dst, int key0, __amdgp
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int i = 0; i < T::N8; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc_k, (lds_ptr_t)(dst + t * T::BYTES + (wave * T::N8 + i) * 1024), 16, voff_k[i],
-          (int)((key0 + 64 * t) * k_ss * 2), 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc_v, (lds_ptr_t)(dst + (2 + t) * T::BYTES + (wave * T::N8 + i) * 1024), 16, voff_v[i],
-          (int)((key0 + 64 * t) * v_ss * 2), 0, 0);
+      dma_load16(rsrc_k, voff_k[i], (int)((key0 + 64 * t) * k_ss * 2), lds_addr_of(dst + t * T::BYTES + (wave * T::N8 + i) * 1024));
+      dma_load16(rsrc_v, voff_v[i], (int)((key0 + 64 * t) * v_ss * 2), lds_addr_of(dst + (2 + t) * T::BYTES + (wave * T::N8 + i) * 1024));
     }
 }
 
@@ -747,8 +764,9 @@ template <int D>
 __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   using T = AttnTile<D>;
   using G = AttnQStage<D>;
-  __shared__ __attribute__((aligned(1024))) char smem[G::LDS];
-  __shared__ uint32_t s_list[ATT_MAX_KB];
+  // one LDS object for the stages and the tile list (see attn_smem_note)
+  __shared__ __attribute__((aligned(1024))) char smem[G::LDS + ATT_MAX_KB * 4];
+  uint32_t* const s_list = (uint32_t*)(smem + G::LDS);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int kg = wave & 3, qh = wave >> 2;
@@ -763,14 +781,14 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   if (light && hq != hkv * rep) return;  // the group's first head does all of them
   const int nheads = light ? rep : 1;
   for (int i = threadIdx.x; i < cnt; i += 512) s_list[i] = p.listT[(int64_t)kb * p.nQb2 + i];
-  const int gk = p.gc[key];
+  int gk = p.gc[key];
 
-  const __amdgpu_buffer_rsrc_t rsrc_q = attn_rsrc(p.Q);
-  const __amdgpu_buffer_rsrc_t rsrc_do = attn_rsrc(p.dO);
+  const dma_rsrc_t rsrc_q = attn_rsrc(p.Q);
+  const dma_rsrc_t rsrc_do = attn_rsrc(p.dO);
   const int arr = wave & 3;
   const void* row_src = arr == 0 ? (const void*)p.lse2 : arr == 1 ? (const void*)p.delta
                         : arr == 2 ? (const void*)p.gc : (const void*)p.pc;
-  const __amdgpu_buffer_rsrc_t rsrc_row = attn_rsrc(row_src);
+  const dma_rsrc_t rsrc_row = attn_rsrc(row_src);
   int voff_q[T::N8], voff_do[T::N8];
   {
     int voff_k[T::N8], voff_v[T::N8];
@@ -807,11 +825,12 @@ __global__ __launch_bounds__(512) void attn_bwd_kv_kernel(AttnBwdParams p) {
   const int krow = 32 * (kg & 1) + n;
 
   const int total = cnt * nheads;
+  pin_loaded(gk);
   if (total > 0) ATTN_ISSUE(0, 0);
   int ti = 0;
   for (int it = 0; it < total; ++it) {
     wait_vmcnt<0>();
-    __syncthreads();
+    barrier_lds_only();
     if (it + 1 < total) ATTN_ISSUE(it + 1, (it + 1) & 1);
     const int entry = __builtin_amdgcn_readfirstlane(s_list[ti]);
     ti = ti + 1 == cnt ? 0 : ti + 1;

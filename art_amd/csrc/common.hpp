@@ -94,4 +94,40 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+// Work-group barrier that waits for this wave's LDS traffic only.  __syncthreads() also carries a
+// fence, for which the compiler drains every outstanding memory operation first (s_waitcnt
+// vmcnt(0)): that would serialise the DMA ring, whose completion is tracked by hand here.
+__device__ __forceinline__ void barrier_lds_only() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+
+// LDS DMA (buffer_load ... lds: 64 lanes x 16 or 4 bytes land at lds_addr + 16 / 4 lane) issued
+// from inline assembly.  Issued through the builtin, the compiler knows that LDS is written
+// behind its back and puts s_waitcnt vmcnt(..) in front of later LDS reads, down to vmcnt(0)
+// once per loop iteration, which drains a multi-stage ring; kernels that track the completion
+// by hand (s_waitcnt vmcnt(n) before the barrier that publishes a stage) keep the instruction
+// out of its sight.  Invisible operations only make the compiler's own waits stricter; the
+// hand-written counts must not have other vector memory operations between issue and wait.
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t dma_rsrc_t;
+__device__ __forceinline__ dma_rsrc_t dma_make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  return dma_rsrc_t{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+}
+__device__ __forceinline__ void dma_load16(dma_rsrc_t rsrc, int voff, int soff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void dma_load4(dma_rsrc_t rsrc, int voff, int soff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
 }  // namespace artk

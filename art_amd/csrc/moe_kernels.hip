@@ -97,43 +97,90 @@ __global__ __launch_bounds__(PERM_CHUNK) void moe_hist_kernel(const int* __restr
 // offsets[e]: first sorted position of expert e; base[b][e]: first sorted
 // position of chunk b's entries of expert e; tile_prefix / blk_prefix: prefix
 // sums of ceil(rows_e / 256) and ceil(rows_e / 16) (work lists of the grouped
-// kernels).  One block of 256 threads.
-__global__ __launch_bounds__(256) void moe_scan_kernel(const int* __restrict__ cnt, int nb, int E,
-                                                       int* __restrict__ offsets,
-                                                       int* __restrict__ base,
-                                                       int* __restrict__ tile_prefix,
-                                                       int* __restrict__ blk_prefix) {
-  __shared__ int tot[MOE_MAX_E];
-  __shared__ int off[MOE_MAX_E + 1];
-  const int e = threadIdx.x;
+// kernels).  One block of 1024 threads: thread (part, e) walks a quarter of the
+// chunks of expert e, eight independent loads at a time.
+constexpr int SCAN_PARTS = 4;
+__global__ __launch_bounds__(SCAN_PARTS * MOE_MAX_E) void moe_scan_kernel(const int* __restrict__ cnt, int nb, int E,
+                                                                          int* __restrict__ offsets,
+                                                                          int* __restrict__ base,
+                                                                          int* __restrict__ tile_prefix,
+                                                                          int* __restrict__ blk_prefix) {
+  __shared__ int part[SCAN_PARTS][MOE_MAX_E];
+  __shared__ int wsum[3][MOE_MAX_E / 64];
+  __shared__ int off[MOE_MAX_E];
+  const int e = threadIdx.x % MOE_MAX_E, pt = threadIdx.x / MOE_MAX_E;
+  const int per = (nb + SCAN_PARTS - 1) / SCAN_PARTS;
+  const int b0 = pt * per, b1 = b0 + per < nb ? b0 + per : nb;
+  int s = 0;
   if (e < E) {
-    int s = 0;
-    for (int b = 0; b < nb; ++b) s += cnt[b * E + e];
-    tot[e] = s;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0, tp = 0, bp = 0;
-    for (int i = 0; i < E; ++i) {
-      off[i] = run;
-      offsets[i] = run;
-      tile_prefix[i] = tp;
-      blk_prefix[i] = bp;
-      run += tot[i];
-      tp += (tot[i] + TILE - 1) / TILE;
-      bp += (tot[i] + 15) / 16;
+    for (int b = b0; b < b1; b += 8) {
+      int v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = b + u < b1 ? cnt[(b + u) * E + e] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
     }
-    off[E] = run;
-    offsets[E] = run;
-    tile_prefix[E] = tp;
-    blk_prefix[E] = bp;
+  }
+  part[pt][e] = s;
+  __syncthreads();
+  // exclusive prefix sums over the experts (threads of part 0: one expert each)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int tot = 0, run = 0, tp = 0, bp = 0;
+  if (pt == 0) {
+    if (e < E)
+#pragma unroll
+      for (int q = 0; q < SCAN_PARTS; ++q) tot += part[q][e];
+    run = tot;
+    tp = (tot + TILE - 1) / TILE;
+    bp = (tot + 15) / 16;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int a = __shfl_up(run, d, 64), t = __shfl_up(tp, d, 64), c = __shfl_up(bp, d, 64);
+      if (lane >= d) {
+        run += a;
+        tp += t;
+        bp += c;
+      }
+    }
+    if (lane == 63) {
+      wsum[0][wave] = run;
+      wsum[1][wave] = tp;
+      wsum[2][wave] = bp;
+    }
+  }
+  __syncthreads();
+  if (pt == 0) {
+    for (int w = 0; w < wave; ++w) {
+      run += wsum[0][w];
+      tp += wsum[1][w];
+      bp += wsum[2][w];
+    }
+    // inclusive sums -> entry e + 1; entry 0 is zero
+    if (e < E) {
+      offsets[e + 1] = run;
+      tile_prefix[e + 1] = tp;
+      blk_prefix[e + 1] = bp;
+      off[e] = run - tot;
+    }
+    if (e == 0) {
+      offsets[0] = 0;
+      tile_prefix[0] = 0;
+      blk_prefix[0] = 0;
+    }
   }
   __syncthreads();
   if (e < E) {
-    int run = off[e];
-    for (int b = 0; b < nb; ++b) {
-      base[b * E + e] = run;
-      run += cnt[b * E + e];
+    int pos = off[e];
+    for (int q = 0; q < pt; ++q) pos += part[q][e];
+    for (int b = b0; b < b1; b += 8) {
+      int v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = b + u < b1 ? cnt[(b + u) * E + e] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (b + u < b1) base[(b + u) * E + e] = pos;
+        pos += v[u];
+      }
     }
   }
 }
@@ -205,12 +252,17 @@ struct MoeTile {
 };
 
 __device__ __forceinline__ MoeTile moe_tile(const MoeGemmParams& p, int t, int n_work) {
+  // Ids run expert by expert and, inside an expert, weight tile by weight tile over its row
+  // tiles: the two or three work-groups that need the same weight tile have neighbouring ids,
+  // start together and read it from HBM once (the L2 of their XCD serves the others); the MT
+  // work-groups that share a row tile are only a few ids apart and still run side by side.
   const int id = xcd_remap(t, n_work);
-  const int rt = id / p.MT;
   MoeTile m;
-  m.mt = id - rt * p.MT;
-  m.e = find_group(p.tile_prefix, p.E, rt);
-  m.row0 = p.offsets[m.e] + (int64_t)(rt - p.tile_prefix[m.e]) * TILE;
+  m.e = find_group(p.tile_prefix, p.E, id / p.MT);
+  const int first = p.tile_prefix[m.e], n_e = p.tile_prefix[m.e + 1] - first;
+  const int local = id - first * p.MT;
+  m.mt = local / n_e;
+  m.row0 = p.offsets[m.e] + (int64_t)(local - m.mt * n_e) * TILE;
   m.row_end = p.offsets[m.e + 1];
   m.nvalid = (int)(m.row_end - m.row0 < TILE ? m.row_end - m.row0 : TILE);
   return m;
@@ -564,7 +616,7 @@ int32_t artk_moe_route(const float* router_logits, int64_t T, int32_t E, int32_t
   ARTK_CHECK_LAUNCH();
   moe_hist_kernel<<<nb, PERM_CHUNK, 0, st>>>(topk_idx, n, E, cnt);
   ARTK_CHECK_LAUNCH();
-  moe_scan_kernel<<<1, 256, 0, st>>>(cnt, nb, E, expert_offsets, base, tile_prefix, blk_prefix);
+  moe_scan_kernel<<<1, SCAN_PARTS * MOE_MAX_E, 0, st>>>(cnt, nb, E, expert_offsets, base, tile_prefix, blk_prefix);
   ARTK_CHECK_LAUNCH();
   moe_scatter_kernel<<<nb, PERM_CHUNK, 0, st>>>(topk_idx, n, E, k, base, perm, inv_perm, row_token);
   ARTK_CHECK_LAUNCH();

@@ -73,13 +73,6 @@ __device__ __forceinline__ bf16x8 st_tr_frag(const char* tile, int lane, int k0,
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// Work-group barrier that waits for this wave's LDS traffic only.  __syncthreads() also carries a
-// fence, for which the compiler drains every outstanding memory operation first (s_waitcnt
-// vmcnt(0)): that would serialise the DMA ring, whose completion is tracked by hand here.
-__device__ __forceinline__ void barrier_lds_only() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // One LDS DMA instruction (64 lanes x 16 bytes land at lds_addr + 16 lane) issued from inline
 // assembly.  Issued through the builtin, the compiler would know that LDS is being written
 // behind its back and put s_waitcnt vmcnt(0) in front of every later LDS read, which drains
