@@ -79,10 +79,12 @@ def attention_rows(q, k, v, group_ids, parent_ids, rows, scale=None, dtype=torch
     Hkv = k.shape[1]
     rep = Hq // Hkv
     scale = 1.0 / math.sqrt(D) if scale is None else scale
-    j = torch.arange(S).unsqueeze(0)
+    dev = q.device  # all inputs on one device (the full-size tests run this restatement on the GPU)
+    j = torch.arange(S, device=dev).unsqueeze(0)
     vis = (j <= rows.unsqueeze(1)) & ((group_ids[rows].unsqueeze(1) == group_ids.unsqueeze(0)) |
                                       (parent_ids[rows].unsqueeze(1) == group_ids.unsqueeze(0)))
-    bias = torch.where(vis, torch.zeros((), dtype=dtype), torch.full((), float("-inf"), dtype=dtype))
+    bias = torch.where(vis, torch.zeros((), dtype=dtype, device=dev),
+                       torch.full((), float("-inf"), dtype=dtype, device=dev))
     qh = q[rows].to(dtype).permute(1, 0, 2)
     kh = k.to(dtype).permute(1, 0, 2).repeat_interleave(rep, 0)
     vh = v.to(dtype).permute(1, 0, 2).repeat_interleave(rep, 0)

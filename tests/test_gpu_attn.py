@@ -196,6 +196,46 @@ def test_attn_full_size_windows(artk_lib, gpu):
     assert torch.equal(out2.float().cpu(), out)
 
 
+def test_attn_bwd_full_size_against_oracle(artk_lib, gpu):
+    """Backward at the full 7B shape (16384 positions, 28 query / 4 key-value heads of 128): dQ, dK and
+    dV of the WHOLE row against the oracle, which runs here on the GPU in fp32, 512 queries at a time
+    (autograd accumulates dK and dV over the chunks), plus the two sums that need no oracle."""
+    print("attention backward S=16384, 28/4 x 128", flush=True)
+    S, Hq, Hkv, D = 16384, 28, 4, 128
+    q, k, v = make_qkv(177, S, Hq, Hkv, D)
+    g = torch.Generator().manual_seed(178)
+    d_out = torch.randn(S, Hq, D, generator=g).to(torch.bfloat16)
+    group, parent = synthetic.packed_row_ids(179, S, 8, 128, 4, 470)   # 8 * 2008 = 16064, rest padding
+    qd, kd, vd, dod = q.to(gpu), k.to(gpu), v.to(gpu), d_out.to(gpu)
+    gd, pd = group.to(gpu), parent.to(gpu)
+    plan = ops.attn_plan(gd, pd)
+    out, lse = ops.attn_fwd(qd, kd, vd, plan)
+    dq, dk, dv = ops.attn_bwd(qd, kd, vd, out, lse, dod, plan)
+    qr = qd.float().requires_grad_(True)
+    kr = kd.float().requires_grad_(True)
+    vr = vd.float().requires_grad_(True)
+    for start in range(0, S, 512):
+        rows = torch.arange(start, start + 512, device=gpu)
+        ref_out, ref_lse = attn_oracle.attention_rows(qr, kr, vr, gd, pd, rows)
+        assert (lse[:, rows] - ref_lse.detach()).abs().max().item() <= 2e-3
+        assert rel_l2(out[rows].float(), ref_out.detach()) <= 1e-2
+        ref_out.backward(dod[rows].float())
+    assert rel_l2(dq.float(), qr.grad) <= 1e-2
+    assert rel_l2(dk.float(), kr.grad) <= 1e-2
+    assert rel_l2(dv.float(), vr.grad) <= 1e-2
+    # per completion block too, so that an error confined to a few rows cannot hide in the norm
+    for lo in range(0, S, 2048):
+        assert rel_l2(dk[lo:lo + 2048].float(), kr.grad[lo:lo + 2048]) <= 1.5e-2
+        assert rel_l2(dv[lo:lo + 2048].float(), vr.grad[lo:lo + 2048]) <= 1.5e-2
+        assert rel_l2(dq[lo:lo + 2048].float(), qr.grad[lo:lo + 2048]) <= 1.5e-2
+    rep = Hq // Hkv
+    want_dv = d_out.double().view(S, Hkv, rep, D).sum((0, 2))            # each softmax row sums to 1
+    got_dv = dv.double().cpu().sum(0)
+    assert ((got_dv - want_dv).norm() / want_dv.norm()).item() <= 1e-2
+    dk64 = dk.double().cpu()                                             # each row of dS sums to 0
+    assert dk64.sum(0).abs().max().item() <= 2.0 ** -8 * dk64.abs().sum(0).max().item()
+
+
 def test_attn_longest_row_windows_and_sums(artk_lib, gpu):
     """The longest row the kernels take (65536 positions, no padding): forward and dQ on windows
     of queries against the oracle, and two sums over the whole row that need no oracle:
