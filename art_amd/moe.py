@@ -66,21 +66,31 @@ class MoELoRAExperts(nn.Module):
         super().__init__()
         self.top_k, self.scaling = top_k, lora_alpha / r
         bf = dict(device=device, dtype=torch.bfloat16)
+        # gate and up read the same rows: they are stored as ONE [E, 2I, H] weight (gate rows first) so
+        # that they run as one grouped product (one pass over x, twice the K length in the
+        # input-gradient product); `gate_weight` / `up_weight` are views of it, not copies
+        self.register_parameter("gate_up_weight", nn.Parameter(
+            0.02 * torch.randn(n_experts, 2 * intermediate, hidden, **bf), requires_grad=False))
+        self.register_parameter("down_weight", nn.Parameter(
+            0.02 * torch.randn(n_experts, hidden, intermediate, **bf), requires_grad=False))
         shapes = {"gate": (intermediate, hidden), "up": (intermediate, hidden), "down": (hidden, intermediate)}
         for name, (o, i) in shapes.items():
-            self.register_parameter(f"{name}_weight", nn.Parameter(
-                0.02 * torch.randn(n_experts, o, i, **bf), requires_grad=False))
             bound = 1.0 / i ** 0.5
             self.register_parameter(f"{name}_lora_A", nn.Parameter(
                 (torch.rand(n_experts, r, i, device=device) * 2 - 1) * bound))
             self.register_parameter(f"{name}_lora_B", nn.Parameter(torch.zeros(n_experts, o, r, device=device)))
-        # gate and up read the same rows: kept as one [E, 2I, H] weight so that they are one
-        # grouped product (one pass over x, twice the K length in the input-gradient product)
-        self.register_parameter("gate_up_weight", nn.Parameter(
-            torch.cat([self.gate_weight.detach(), self.up_weight.detach()], 1).contiguous(),
-            requires_grad=False))
         self.intermediate = intermediate
         self._wt = {}
+
+    @property
+    def gate_weight(self) -> torch.Tensor:
+        """[E, I, H] view of the gate rows of gate_up_weight."""
+        return self.gate_up_weight[:, :self.intermediate]
+
+    @property
+    def up_weight(self) -> torch.Tensor:
+        """[E, I, H] view of the up rows of gate_up_weight."""
+        return self.gate_up_weight[:, self.intermediate:]
 
     def _transposed(self, name):
         w = getattr(self, f"{name}_weight")

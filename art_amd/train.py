@@ -249,9 +249,22 @@ def get_compute_loss_fn(trainer) -> Callable[..., torch.Tensor]:
         assert (
             seq_len % chunk_size == 0
         ), f"Sequence length ({seq_len}) must be evenly divisible by chunk size ({chunk_size})"
-        attn_bias = calculate_attn_bias(batch_size, seq_len, device, inputs["group_ids"],
-                                        inputs["parent_ids"], autocast_dtype)
+        if _config.get("packed_attention_plans", False):
+            # opt-in (no counterpart in the reference): the model's attention layers call
+            # art_amd.attention.packed_attention and take, as `causal_mask`, one plan per packed row
+            # made from the ids; the dense [B, S, S] bias (2 S^2 bytes per row) is never built
+            attn_bias = [ops.attn_plan(inputs["group_ids"][b].contiguous(), inputs["parent_ids"][b].contiguous())
+                         for b in range(batch_size)]
+        else:
+            attn_bias = calculate_attn_bias(batch_size, seq_len, device, inputs["group_ids"],
+                                            inputs["parent_ids"], autocast_dtype)
         lm_head = trainer.model.get_output_embeddings().weight  # [V, H]
+        if lm_head.requires_grad:
+            # the fused step treats lm_head as frozen (LoRA on the attention / MLP projections only, the
+            # reference's set-up): it computes no gradient for it, where the reference's autograd would
+            raise NotImplementedError(
+                "the output embedding is trainable (requires_grad=True, e.g. through modules_to_save): "
+                "the fused GRPO step computes no gradient for lm_head; freeze it or use the reference loss")
         os.environ["UNSLOTH_RETURN_HIDDEN_STATES"] = "1"
 
         ref_logprobs = None

@@ -14,7 +14,7 @@ import torch
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
 import grpo_oracle  # noqa: E402
 
-from art_amd import synthetic  # noqa: E402
+from art_amd import ops, synthetic  # noqa: E402
 from art_amd.train import get_compute_loss_fn  # noqa: E402
 
 pytestmark = pytest.mark.gpu
@@ -45,6 +45,7 @@ class TinyModel(torch.nn.Module):
             self.use_adapter = True
 
     def forward(self, input_ids, causal_mask):
+        self.last_mask = causal_mask
         h = self.emb[input_ids]
         if self.use_adapter:
             h = h + self.adapter[input_ids]
@@ -77,6 +78,7 @@ def test_compute_loss_patch(artk_lib, gpu, beta):
               "logprobs": case.logprobs, "advantages": case.advantages, "weights": case.weights,
               "config": types.SimpleNamespace(learning_rate=3e-6, beta=beta),
               "_config": {"logprob_calculation_chunk_size": 256, "epsilon": 0.2}}
+    inputs_backup = {k: v for k, v in inputs.items() if k not in ("config", "_config")}
     loss = compute_loss(model, inputs)
     loss.backward()
 
@@ -101,6 +103,23 @@ def test_compute_loss_patch(artk_lib, gpu, beta):
     bad = dict(inputs, config=inputs_config(beta), _config={"logprob_calculation_chunk_size": 300})
     with pytest.raises(AssertionError):
         compute_loss(model, bad)
+    # the dense bias by default; with the opt-in the model gets one attention plan per row instead
+    assert torch.is_tensor(model.last_mask) and model.last_mask.shape == (1, S, S)
+    again = {k: v for k, v in inputs_backup.items()}
+    again["config"] = inputs_config(beta)
+    again["_config"] = {"logprob_calculation_chunk_size": 256, "epsilon": 0.2, "packed_attention_plans": True}
+    loss2 = compute_loss(model, again)
+    assert isinstance(model.last_mask, list) and len(model.last_mask) == 1
+    assert isinstance(model.last_mask[0], ops.AttnPlan) and model.last_mask[0].S == S
+    assert loss2.item() == loss.item()
+    # a trainable output embedding is refused: the fused step computes no gradient for it
+    model.head.weight.requires_grad_(True)
+    try:
+        with pytest.raises(NotImplementedError, match="lm_head"):
+            compute_loss(model, dict(inputs_backup, config=inputs_config(beta),
+                                     _config={"logprob_calculation_chunk_size": 256}))
+    finally:
+        model.head.weight.requires_grad_(False)
 
 
 def inputs_config(beta):

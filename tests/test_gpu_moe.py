@@ -176,6 +176,9 @@ def test_moe_block_autograd(artk_lib, gpu):
     ref = moe_oracle.route(logits.cpu(), k)
     xr = x.detach().cpu().float().requires_grad_(True)
     P = {n: p.detach().cpu().float().requires_grad_(p.requires_grad) for n, p in mod.named_parameters()}
+    assert "gate_weight" not in P and "up_weight" not in P    # one stored weight; gate / up are views of it
+    assert mod.gate_weight.data_ptr() == mod.gate_up_weight.data_ptr()
+    P["gate_weight"], P["up_weight"] = P["gate_up_weight"][:, :I], P["gate_up_weight"][:, I:]
     rows = xr[ref["row_token"]]
     off = ref["offsets"]
     s = mod.scaling
