@@ -29,11 +29,11 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E peak
 # (FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None until
 # measured for the workload.  Source: profiles/lmhead_fwd_c3_pmc.md
 TRAFFIC_BYTES = {"c3": 2.05e10, "c1": None}
-# moe_gemm_kernel, mean HBM bytes per launch of the separate-projection step (FETCH_SIZE x 2 KiB + WRITE_SIZE
-# x 1 KiB, the factors a 1 GiB copy gives): (3 x 723 + 3 x 586) / 6 MB read + (3 x 101 + 3 x 269) / 6 MB written
-MOE_TRAFFIC_BYTES = 8.4e8
-MOE_TRAFFIC_SOURCE = ("profiles/moe_c5_kernel_trace.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run, "
-                      "separate projections, scaled by a 1 GiB copy; not measured in this run)")
+# moe_gemm_kernel, mean bytes per launch over the 4 launches of the step with gate|up fused (FETCH_SIZE x 2 KiB +
+# WRITE_SIZE x 1 KiB, the factors a 1 GiB copy gives): 949 MB read + 210 MB written
+MOE_TRAFFIC_BYTES = 1.16e9
+MOE_TRAFFIC_SOURCE = ("profiles/moe_c5_kernel_trace.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of "
+                      "this command, scaled by a 1 GiB copy; not measured in this run)")
 TRAFFIC_SOURCE = {"c3": "profiles/lmhead_fwd_c3_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier "
                         "run of this command, scaled by a 1 GiB copy; not measured in this run)"}
 
