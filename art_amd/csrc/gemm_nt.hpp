@@ -28,6 +28,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace artk {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -209,8 +211,8 @@ struct TileLoaders {
 //                current stage is free, and the next stage has landed
 //   step 3     : MFMAs while step 0 of the next stage is read; the first half
 //                of the DMA for the stage after next goes into the freed buffer
-// The loop body has no branches: past the end, the DMA re-fetches the last
-// stage into the idle buffer and the fragment prefetch reads values nobody uses.
+// The loop body has no branches; the last two K-steps are peeled off without the DMA
+// that would reach past the end of the K range.
 __device__ __forceinline__ void gemm_tile_run_pinned(TileAcc<4>& acc, char* smem, const TileLoaders<4>& L);
 
 template <int NI>
@@ -240,28 +242,30 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
   const int q_wave_off = OPER_STAGE_BYTES + wn * (32 * NI) * 128;
 
   const int nk = (k_end - k_begin) / BK;
-  const int k_last = k_end - BK;
 
   constexpr int EARLY = NI;  // DMA instructions per operand issued right after the barrier
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  {
-    int k1 = k_begin + BK < k_last ? k_begin + BK : k_last;
-    lp.template issue<0, EARLY>(smem + STAGE_BYTES, wave, k1);
-    lq.template issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k1);
+  if (nk > 1) {
+    lp.template issue<0, EARLY>(smem + STAGE_BYTES, wave, k_begin + BK);
+    lq.template issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
   }
   Frags<NI> f0, f1;
   load_frags(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
 
-  for (int kt = 0; kt < nk; ++kt) {
+  // One K-step.  LATE: the second half of stage kt + 1 is still to be issued (false in the last
+  // K-step); AHEAD: the first half of stage kt + 2 goes out after the barrier (false in the last
+  // two).  The last K-steps are peeled off with those flags cleared instead of re-fetching the
+  // last stage: on a 12-step K loop the re-fetches were an eighth of the traffic into LDS.
+  auto k_step = [&](int kt, auto late_tag, auto ahead_tag) {
+    constexpr bool LATE = decltype(late_tag)::value, AHEAD = decltype(ahead_tag)::value;
     char* cur = smem + (kt & 1) * STAGE_BYTES;
     char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
     const char* sp = cur + p_wave_off;
     const char* sq = cur + q_wave_off;
 
-    {
-      int k1 = k_begin + (kt + 1) * BK;
-      k1 = k1 < k_last ? k1 : k_last;
+    if constexpr (LATE) {
+      const int k1 = k_begin + (kt + 1) * BK;
       lp.template issue<EARLY, DI>(nxt, wave, k1);
       lq.template issue<EARLY, DI>(nxt + OPER_STAGE_BYTES, wave, k1);
     }
@@ -272,27 +276,28 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
     load_frags(f1, sp, sq, off[3]);
     mma_frags(acc, f0);
     // Interleave: 3 steps of 4*NI MFMAs, 3*(4+NI) LDS reads, 2*(DI-EARLY) DMA issues.
+    constexpr int NLATE = LATE ? 2 * (DI - EARLY) : 0;
     if constexpr (NI == 4) {
 #pragma unroll
-      for (int i = 0; i < 2 * (DI - EARLY); ++i) {
+      for (int i = 0; i < NLATE; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // 2 MFMA
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
       }
 #pragma unroll
-      for (int i = 0; i < 24 - 2 * (DI - EARLY); ++i) {
+      for (int i = 0; i < 24 - NLATE; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 2 * (DI - EARLY); ++i) {
+      for (int i = 0; i < NLATE; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 DMA issue
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
       }
 #pragma unroll
-      for (int i = 0; i < 18 - 2 * (DI - EARLY); ++i) {
+      for (int i = 0; i < 18 - NLATE; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -302,10 +307,12 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
 
-    int k2 = k_begin + (kt + 2) * BK;
-    k2 = k2 < k_last ? k2 : k_last;
-    lp.template issue<0, EARLY>(cur, wave, k2);
-    lq.template issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
+    if constexpr (AHEAD) {
+      const int k2 = k_begin + (kt + 2) * BK;
+      lp.template issue<0, EARLY>(cur, wave, k2);
+      lq.template issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
+    }
+    // (after the last K-step this reads the idle stage: values nobody uses)
     load_frags(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
     mma_frags(acc, f1);
     // 4*NI MFMA, 4+NI LDS reads, 2*EARLY DMA issues
@@ -313,20 +320,25 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        if (i < EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        if (AHEAD && i < EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 6; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (AHEAD && i < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     }
-  }
-  // Drain the redundant tail DMA before the caller reuses or releases LDS.
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+  for (int kt = 0; kt < nk - 2; ++kt) k_step(kt, yes{}, yes{});
+  if (nk > 1) k_step(nk - 2, yes{}, no{});
+  k_step(nk - 1, no{}, no{});
+  // Nothing is outstanding here; the caller may reuse or release LDS.
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
 }
