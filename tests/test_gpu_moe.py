@@ -110,6 +110,42 @@ def test_grouped_lora_matches_oracle(artk_lib, gpu, T, H, I, E, k, use_gather):
     assert rel_l2(dB.cpu(), dB0) <= TOL
 
 
+@pytest.mark.parametrize("use_gather", [True, False])
+def test_grouped_lora_with_empty_experts(artk_lib, gpu, use_gather):
+    """Experts that no token chose: their dA_e and dB_e are exactly zero, the others match the oracle
+    (the one-pass backward gives every expert its own slab of rows, here some of them empty, one of
+    them longer than a 128-row tile and the first and last expert among the empty ones)."""
+    print(f"moe grouped, empty experts, gather={use_gather}", flush=True)
+    T, H, I, E, k = 320, 128, 192, 16, 2
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(T, E, generator=g)
+    dead = [0, 3, 4, 5, 15]
+    logits[:, dead] = float("-inf")
+    logits[:200, 7] += 8.0                      # expert 7 gets at least 200 rows
+    r, ref = check_routing(logits, k, gpu)
+    off = ref["offsets"]
+    assert all(off[e + 1] == off[e] for e in dead) and off[8] - off[7] >= 200
+    n_rows = T * k
+    x = torch.randn(T if use_gather else n_rows, H, generator=g).to(torch.bfloat16)
+    W, A, B = make_experts(E, I, H, 8, 9)
+    up = torch.randn(n_rows, I, generator=g).to(torch.bfloat16)
+    y0, dx0, dA0, dB0 = moe_oracle.grouped_lora_grads(
+        x, ref["row_token"] if use_gather else None, W, A, B, 2.0, off, up)
+    gather = r.row_token if use_gather else None
+    y, xa = ops.moe_lora_grouped_fwd(x.to(gpu), gather, W.to(gpu), A.to(gpu), B.to(gpu), 2.0, r)
+    dx, dA, dB = ops.moe_lora_grouped_bwd(up.to(gpu), x.to(gpu), gather, ops.transpose_batched(W.to(gpu)),
+                                          A.to(gpu), B.to(gpu), xa, 2.0, r)
+    assert rel_l2(y.cpu().float(), y0) <= TOL
+    if use_gather:
+        dx = dx[r.inv_perm.long()].view(T, k, H).float().sum(1)
+    assert rel_l2(dx.cpu().float(), dx0) <= TOL
+    assert rel_l2(dA.cpu(), dA0) <= TOL and rel_l2(dB.cpu(), dB0) <= TOL
+    for e in dead:
+        assert dA[e].abs().max().item() == 0.0 and dB[e].abs().max().item() == 0.0
+    for e in (7, 8):
+        assert rel_l2(dA[e].cpu(), dA0[e]) <= TOL and rel_l2(dB[e].cpu(), dB0[e]) <= TOL
+
+
 def test_config5_gate_projection_full_size(artk_lib, gpu):
     """Benchmark config 5: 8192 tokens, hidden 2048, 128 experts, top-8, gate [768,2048]."""
     print("moe config5 gate projection", flush=True)
