@@ -62,7 +62,7 @@ struct Workspace {
 // ---- optional per-kernel timing with HIP events on the launch stream ---------
 // Off by default. When on, the launch helpers bracket each dominant kernel with
 // two events; artk_profile_collect() (after the caller synchronised) sums them.
-enum ProfKind { PROF_LMHEAD_FWD = 0, PROF_DHIDDEN_GEMM = 1, PROF_SOFTMAX_GRAD = 2,
+enum ProfKind { PROF_LMHEAD_FWD = 0, PROF_DHIDDEN_GEMM = 1, PROF_TARGET_REF = 2,
                 PROF_LORA_GEMM = 3, PROF_MOE_GEMM = 4, PROF_ATTN_FWD = 5, PROF_ATTN_BWD_KV = 6,
                 PROF_ATTN_BWD_Q = 7, PROF_KINDS = 8 };
 void prof_begin(int kind, hipStream_t st);

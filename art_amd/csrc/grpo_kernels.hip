@@ -76,7 +76,8 @@ struct FwdParams {
   int shift;
   float2* part;         // [2*VT][Tc]  (max, sumexp)
   float* sel;           // [Tc]        selected logit (pre-filled with NaN)
-  uint16_t* stash;      // [Tc,V] bf16 logits or nullptr
+  uint16_t* stash;      // [Tc,V] bf16 or nullptr: exp(logit - ref[row]) of the rows the backward reads
+  const float* ref;     // [Tc] reference logit of each row (stash only): the target's own logit
   const uint8_t* need;  // [Tc] rows of the stash that the backward will read; nullptr: all
   int VT, TT;
 };
@@ -162,6 +163,7 @@ __device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, 
       if (!__any(want)) continue;
       if (want) {
         uint16_t* row = p.stash + (int64_t)col[ni] * p.V;
+        const float nref = -p.ref[col[ni]] * LOG2E;
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
@@ -170,7 +172,8 @@ __device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, 
             if (v < p.V) {
               bf16x4 o;
 #pragma unroll
-              for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
+              for (int e = 0; e < 4; ++e)
+                o[e] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][q * 4 + e], LOG2E, nref));
               *(bf16x4*)(row + v) = o;
             }
           }
@@ -552,39 +555,48 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restr
   }
 }
 
-// K3b: in-place softmax gradient on the bf16 logits scratch, active rows only:
-//   P[t,v] = coef[t] * ( [v == y_t] - exp(z[t,v] - lse[t]) )
-// One block per active row.
-__global__ __launch_bounds__(256) void softmax_grad_kernel(uint16_t* __restrict__ stash, int64_t V,
-                                                           const float* __restrict__ lse,
-                                                           const float* __restrict__ coef,
-                                                           const int64_t* __restrict__ ids,
-                                                           ChunkRows rows, int64_t S, int shift,
-                                                           const int* __restrict__ active_idx,
-                                                           const int* __restrict__ sched) {
-  if ((int)blockIdx.x >= sched[0]) return;
-  const int64_t r = active_idx[blockIdx.x];
-  uint4* row = (uint4*)(stash + r * V);
-  const int nvec = (int)(V >> 3);
-  const float c = coef[r];
-  const int64_t y = target_id(ids, rows.token((int)r), S, shift);
-  const float nl = -lse[r] * LOG2E;
-  for (int i = threadIdx.x; i < nvec; i += 256) {
-    uint4 x = row[i];
-    uint32_t w[4] = {x.x, x.y, x.z, x.w};
-    const int64_t v0 = (int64_t)i * 8;
+// K0 (before the forward of a chunk the backward will read): ref[r] = logit of row r's own
+// target, hidden[token(r)] . lm_head[y_r], in fp32; 0 for rows the backward does not need or
+// whose target is not a vocabulary id.  The forward stashes exp(logit - ref[r]) instead of the
+// logit: softmax is invariant to the shift, the target was sampled from (nearly) this
+// distribution, so its logit is a reference within a few tens of nats of the row's maximum,
+// and bf16 has the exponent range of fp32 — exp(z - ref) is representable unless a logit
+// exceeds the target's by 88 nats, i.e. unless the sampled token has probability below
+// e^-88 under the current policy; such a row's d_hidden comes out as inf / NaN, not as a
+// silently wrong number.  With the exponentials in the stash the softmax gradient needs no
+// pass of its own: d_hidden[t] = coef_t (W[y_t] - exp(ref_t - lse_t) sum_v e[t,v] W[v]),
+// the sum being the GEMM K4 and the rest the epilogue of K5.  (A stash of logits needed a
+// 2 x [Tc_active, V] read-modify-write between K2 and K4 to turn them into gradients.)
+// One wave per row.
+__global__ __launch_bounds__(256) void target_ref_kernel(const uint16_t* __restrict__ hidden,
+                                                         const uint16_t* __restrict__ W,
+                                                         const int64_t* __restrict__ ids, ChunkRows rows,
+                                                         const uint8_t* __restrict__ need, int64_t S,
+                                                         int shift, int64_t V, int64_t H,
+                                                         float* __restrict__ ref) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows.n()) return;
+  float s = 0.f;
+  const int64_t y = target_id(ids, rows.token(r), S, shift);
+  if ((need == nullptr || need[r] != 0) && y >= 0 && y < V) {
+    // `hidden` starts at the chunk's first row when the rows are dense, at position 0 when they
+    // are gathered
+    const uint16_t* h = hidden + (int64_t)(rows.row_token ? rows.token(r) : r) * H;
+    const uint16_t* w = W + y * H;
+    for (int64_t k = lane * 8; k < H; k += 512) {
+      const uint4 a = *(const uint4*)(h + k), b = *(const uint4*)(w + k);
+      const uint32_t av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float z0 = __uint_as_float(w[e] << 16);
-      float z1 = __uint_as_float(w[e] & 0xffff0000u);
-      float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(z0, LOG2E, nl));
-      float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(z1, LOG2E, nl));
-      float g0 = c * ((v0 + 2 * e == y ? 1.f : 0.f) - p0);
-      float g1 = c * ((v0 + 2 * e + 1 == y ? 1.f : 0.f) - p1);
-      w[e] = (uint32_t)f32_to_bf16(g0) | ((uint32_t)f32_to_bf16(g1) << 16);
+      for (int e = 0; e < 4; ++e) {
+        s = __builtin_fmaf(__uint_as_float(av[e] << 16), __uint_as_float(bv[e] << 16), s);
+        s = __builtin_fmaf(__uint_as_float(av[e] & 0xffff0000u), __uint_as_float(bv[e] & 0xffff0000u), s);
+      }
     }
-    row[i] = make_uint4(w[0], w[1], w[2], w[3]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
   }
+  if (lane == 0) ref[r] = s;
 }
 
 // ----------------------------------------------------------------------------
@@ -644,13 +656,19 @@ __global__ __launch_bounds__(nthreads<BWD_NI>()) void dhidden_gemm_kernel(BwdPar
   }
 }
 
-// K5: d_hidden row of chunk row r = bf16(sum over splits of partial[active slot
-// of r]) or 0 for inactive rows; 4 elements per thread.  `out` is the whole
-// batch's d_hidden, indexed by position.
+// K5: d_hidden row of chunk row r: 0 for inactive rows, else
+//   bf16( coef_r * ( W[y_r] - exp(ref_r - lse_r) * G ) ),  G = sum over splits of partial[active slot of r]
+// (G = sum_v exp(z[r,v] - ref_r) W[v], see target_ref_kernel); 4 elements per thread.  `out` is
+// the whole batch's d_hidden, indexed by position.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
                                                             const int* __restrict__ pos,
                                                             const int* __restrict__ sched,
-                                                            ChunkRows rows, int64_t H,
+                                                            ChunkRows rows, int64_t H, int64_t V,
+                                                            const float* __restrict__ coef,
+                                                            const float* __restrict__ lse,
+                                                            const float* __restrict__ ref,
+                                                            const int64_t* __restrict__ ids, int64_t S,
+                                                            int shift, const uint16_t* __restrict__ W,
                                                             uint16_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t h4 = H / 4;
@@ -663,6 +681,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     const int64_t rows_per_split = (int64_t)sched[1] * TILE;
     for (int k = 0; k < nsplit; ++k)
       s += ((const floatx4*)(partial + ((int64_t)k * rows_per_split + pr) * H))[c];
+    const float cf = coef[r];
+    const float scale = __builtin_amdgcn_exp2f((ref[r] - lse[r]) * LOG2E);
+    const int64_t y = target_id(ids, rows.token((int)r), S, shift);
+    floatx4 w = {0.f, 0.f, 0.f, 0.f};
+    if (y >= 0 && y < V) {
+      const uint2 wv = *(const uint2*)(W + y * H + c * 4);
+      w[0] = __uint_as_float(wv.x << 16);
+      w[1] = __uint_as_float(wv.x & 0xffff0000u);
+      w[2] = __uint_as_float(wv.y << 16);
+      w[3] = __uint_as_float(wv.y & 0xffff0000u);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] = cf * (w[e] - scale * s[e]);
   }
   bf16x4 o;
 #pragma unroll
@@ -808,13 +839,21 @@ static ChunkRows dense_rows(int64_t t0, int64_t n) {
   return r;
 }
 
-// Launch K1 (+ NaN pre-fill of sel) and K2 for the rows of one chunk.  `logprob`
+// Launch K0 (when the chunk is stashed), K1 (+ NaN pre-fill of sel) and K2 for the rows of one chunk.  `logprob`
 // (may be null) is the whole batch's array; `lse_chunk` is indexed by chunk row.
 static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const int64_t* ids,
                                 int shift, const ChunkRows& rows, int64_t S, int64_t V, int64_t H,
-                                float2* part, float* sel, uint16_t* stash, const uint8_t* need,
+                                float2* part, float* sel, uint16_t* stash, float* ref, const uint8_t* need,
                                 float* logprob, float* lse_chunk, hipStream_t st) {
   const int64_t Tc = rows.cap;
+  if (stash) {
+    prof_begin(PROF_TARGET_REF, st);
+    target_ref_kernel<<<(unsigned)((Tc + 3) / 4), 256, 0, st>>>(
+        (const uint16_t*)(rows.row_token ? hidden : (const void*)((const char*)hidden + rows.t0 * H * 2)),
+        (const uint16_t*)lm_head, ids, rows, need, S, shift, V, H, ref);
+    prof_end(PROF_TARGET_REF, st);
+    ARTK_CHECK_LAUNCH();
+  }
   FwdParams p;
   p.hidden = rows.row_token ? hidden : (const void*)((const char*)hidden + rows.t0 * H * 2);
   p.W = lm_head;
@@ -828,6 +867,7 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   p.part = part;
   p.sel = sel;
   p.stash = stash;
+  p.ref = ref;
   p.need = need;
   p.VT = (int)((V + TILE - 1) / TILE);
   p.TT = (int)((Tc + TILE - 1) / TILE);
@@ -864,22 +904,17 @@ struct BwdScratch {
   int* sched;
 };
 
-// Launch K3a, K3b, K4, K5 for one chunk whose bf16 logits are in `stash`.
+// Launch K3a, K4, K5 for one chunk whose exponentials (see target_ref_kernel) are in `stash`.
 // `d_hidden` is the whole batch's gradient, indexed by position.
-static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const int64_t* ids,
+static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head, const void* lm_head_t, const int64_t* ids,
                                 int shift, const ChunkRows& rows, int64_t S, int64_t V, int64_t H,
-                                const float* lse_chunk, const float* coef_chunk, const BwdScratch& sc,
-                                uint16_t* d_hidden, hipStream_t st) {
+                                const float* lse_chunk, const float* coef_chunk, const float* ref_chunk,
+                                const BwdScratch& sc, uint16_t* d_hidden, hipStream_t st) {
   const int64_t Tc = rows.cap;
   const int HT = (int)((H + TILE - 1) / TILE);
   const int TT = (int)((Tc + TILE - 1) / TILE);
   compact_rows_kernel<<<1, 1024, 0, st>>>(coef_chunk, rows, HT, (int)(V / BK), (int)sc.part_rows,
                                           num_cus(), sc.active_idx, sc.pos, sc.sched);
-  ARTK_CHECK_LAUNCH();
-  prof_begin(PROF_SOFTMAX_GRAD, st);
-  softmax_grad_kernel<<<(unsigned)Tc, 256, 0, st>>>(stash, V, lse_chunk, coef_chunk, ids, rows, S, shift,
-                                                    sc.active_idx, sc.sched);
-  prof_end(PROF_SOFTMAX_GRAD, st);
   ARTK_CHECK_LAUNCH();
   BwdParams b;
   b.Wt = lm_head_t;
@@ -898,8 +933,9 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head_t, const in
   prof_end(PROF_DHIDDEN_GEMM, st);
   ARTK_CHECK_LAUNCH();
   const int64_t n4 = Tc * H / 4;
-  splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(sc.partial, sc.pos, sc.sched, rows,
-                                                                     H, d_hidden);
+  splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(
+      sc.partial, sc.pos, sc.sched, rows, H, V, coef_chunk, lse_chunk, ref_chunk, ids, S, shift,
+      (const uint16_t*)lm_head, d_hidden);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -970,15 +1006,16 @@ int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t*
     set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
     return ARTK_ERR_WORKSPACE_TOO_SMALL;
   }
-  return launch_fwd_chunk(hidden, lm_head, ids, shift, dense_rows(0, T), S, V, H, part, sel, nullptr,
+  return launch_fwd_chunk(hidden, lm_head, ids, shift, dense_rows(0, T), S, V, H, part, sel, nullptr, nullptr,
                           nullptr, logprob, lse, (hipStream_t)stream);
 }
 
 // Scratch of one chunk of Tc positions carved out of the caller's workspace.
 struct ChunkScratch {
-  uint16_t* stash;  // [Tc,V] bf16 logits, then softmax gradient
+  uint16_t* stash;  // [Tc,V] bf16 exp(logit - ref) of the rows the backward reads
   float2* part;     // [2*VT][Tc]
   float* sel;       // [Tc]
+  float* ref;       // [Tc] reference logit per chunk row (target_ref_kernel)
   uint8_t* need;    // [Tc]
   BwdScratch bwd;
   float *lse, *coef;            // [Tc] each, by chunk row (fused op only)
@@ -995,6 +1032,7 @@ static void carve(Workspace& ws, int64_t T, int64_t V, int64_t H, int64_t Tc, bo
   c.stash = ws.take<uint16_t>((size_t)(Tc * V));
   c.part = ws.take<float2>((size_t)(2 * VT * Tc));
   c.sel = ws.take<float>((size_t)Tc);
+  c.ref = ws.take<float>((size_t)Tc);
   c.need = ws.take<uint8_t>((size_t)Tc);
   c.bwd.part_rows = bwd_part_rows(Tc, H, V);
   c.bwd.partial = ws.take<float>((size_t)c.bwd.part_rows * H);
@@ -1083,11 +1121,11 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
     need_from_grad_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(grad_logprob + t0, n, c.need);
     ARTK_CHECK_LAUNCH();
     const ChunkRows rows = dense_rows(t0, n);
-    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, rows, S, V, H, c.part, c.sel, c.stash, c.need,
+    rc = launch_fwd_chunk(hidden, lm_head, ids, shift, rows, S, V, H, c.part, c.sel, c.stash, c.ref, c.need,
                           nullptr, c.lse_tmp, st);
     if (rc) return rc;
-    rc = launch_bwd_chunk(c.stash, lm_head_t, ids, shift, rows, S, V, H, lse + t0, grad_logprob + t0,
-                          c.bwd, (uint16_t*)d_hidden, st);
+    rc = launch_bwd_chunk(c.stash, lm_head, lm_head_t, ids, shift, rows, S, V, H, lse + t0, grad_logprob + t0,
+                          c.ref, c.bwd, (uint16_t*)d_hidden, st);
     if (rc) return rc;
   }
   return ARTK_OK;
@@ -1249,7 +1287,7 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
                                                                            ref, t0, n, S, 1, c.need);
       ARTK_CHECK_LAUNCH();
     }
-    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, rows, S, V, H, c.part, c.sel, c.stash,
+    rc = launch_fwd_chunk(hidden, lm_head, tokens, 1, rows, S, V, H, c.part, c.sel, c.stash, c.ref,
                           skip ? nullptr : c.need, logprob, c.lse, st);
     if (rc) return rc;
     LossParams p;
@@ -1271,7 +1309,7 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
     p.coef = c.coef;
     grpo_loss_tok_kernel<<<(unsigned)((rows.cap + 255) / 256), 256, 0, st>>>(p);
     ARTK_CHECK_LAUNCH();
-    rc = launch_bwd_chunk(c.stash, lm_head_t, tokens, 1, rows, S, V, H, c.lse, c.coef, c.bwd,
+    rc = launch_bwd_chunk(c.stash, lm_head, lm_head_t, tokens, 1, rows, S, V, H, c.lse, c.coef, c.ref, c.bwd,
                           (uint16_t*)d_hidden, st);
     if (rc) return rc;
   }

@@ -637,7 +637,7 @@ def adamw8bit_step(p, g, state1, state2, absmax1, absmax2, qmap1, qmap2, p_bf16,
 # -----------------------------------------------------------------------------
 # per-kernel timing
 # -----------------------------------------------------------------------------
-(PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_SOFTMAX_GRAD, PROF_LORA_GEMM, PROF_MOE_GEMM, PROF_ATTN_FWD,
+(PROF_LMHEAD_FWD, PROF_DHIDDEN_GEMM, PROF_TARGET_REF, PROF_LORA_GEMM, PROF_MOE_GEMM, PROF_ATTN_FWD,
  PROF_ATTN_BWD_KV, PROF_ATTN_BWD_Q) = range(8)
 
 

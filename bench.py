@@ -1010,7 +1010,7 @@ def main():
     dt_profiled = time.perf_counter() - t0
     fwd_ms, fwd_n = ops.profile_collect(ops.PROF_LMHEAD_FWD)
     bwd_ms, bwd_n = ops.profile_collect(ops.PROF_DHIDDEN_GEMM)
-    sm_ms, sm_n = ops.profile_collect(ops.PROF_SOFTMAX_GRAD)
+    sm_ms, sm_n = ops.profile_collect(ops.PROF_TARGET_REF)
     ops.profile_enable(False)
     mask_count = int(out[0][3].item())
     # positions whose loss coefficient is non-zero (masked in, non-zero advantage, unclipped):
@@ -1110,7 +1110,7 @@ def main():
         "kernels": {
             "dhidden_gemm_kernel": {"launch_ms": bwd_launch_ms, "tflops": bwd_achieved,
                                     "frac": bwd_achieved / PEAK_BF16_TFLOPS},
-            "softmax_grad_kernel": {"launch_ms": sm_ms / max(sm_n, 1)},
+            "target_ref_kernel": {"launch_ms": sm_ms / max(sm_n, 1)},
         },
     }
     assert t_active == t_active_dense

@@ -120,8 +120,12 @@ int32_t artk_grpo_loss_static(const float* new_logprob, const float* old_logprob
  * Replaces: the body of compute_loss, src/art/local/train.py:76-151, plus the
  *   backward that HF Trainer.training_step triggers on its result.
  * Per chunk of `chunk_tokens` positions: lm_head GEMM with online log-sum-exp
- * and target gather (bf16 logits of the chunk go to a bounded scratch), loss
- * coefficients, softmax-gradient in place, d_hidden GEMM against lm_head_t.
+ * and target gather (for the rows the backward will read, exp(logit - the
+ * target's logit) goes to a bounded bf16 scratch), loss coefficients, d_hidden
+ * GEMM of those exponentials against lm_head_t, softmax scaling and one-hot
+ * term in its reduction.  A row whose target logit lies more than 88 nats under
+ * the row's largest logit (a sampled token of probability < e^-88) overflows the
+ * scratch: its d_hidden row is inf / NaN.
  *   tokens int64 [T], old_logprob/advantages/weights f32 [T], mask u8 [T]:
  *     the un-shifted PackedTensors rows (src/art/local/pack.py:13-21);
  *     the shift of train.py:79,112-117 is applied by index arithmetic.
@@ -383,7 +387,7 @@ int32_t artk_lora_linear_bwd_nf4(const void* g, const void* x, const artk_nf4_t*
  * ------------------------------------------------------------------------- */
 #define ARTK_PROF_LMHEAD_FWD 0
 #define ARTK_PROF_DHIDDEN_GEMM 1
-#define ARTK_PROF_SOFTMAX_GRAD 2
+#define ARTK_PROF_TARGET_REF 2 /* the reference-logit pre-pass of a stashed chunk */
 #define ARTK_PROF_LORA_GEMM 3
 #define ARTK_PROF_MOE_GEMM 4
 #define ARTK_PROF_ATTN_FWD 5
