@@ -109,6 +109,58 @@ def test_fused_matches_oracle(artk_lib, gpu, T, H, V, n_traj, chunk_tokens):
     assert hidden.grad[0][~m.to(gpu)].abs().max().item() == 0.0
 
 
+def test_fused_wide_logit_range(artk_lib, gpu):
+    """Peaked distributions: logits spread over +-35 nats, targets up to ~65 nats under their row's maximum.
+    The backward works on exp(logit - target logit) in bf16, which has to hold over that range."""
+    T, H, V = 512, 256, 8192
+    case = synthetic.make_grpo_case("w", 31, T, H, V, 4, 4, 0.5)
+    case.hidden = (case.hidden.float() * 25.0).to(torch.bfloat16)
+    ref = oracle_case(case, T)
+    logits = case.hidden[0].float() @ case.lm_head.float().t()
+    nxt = grpo_oracle.shift_tensor(case.tokens, 0)[0]
+    gap = logits.max(-1).values - logits.gather(1, nxt.view(-1, 1)).squeeze(1)
+    assert 40.0 < gap.max().item() < 80.0
+    hidden = case.hidden.to(gpu).requires_grad_(True)
+    loss, metrics, logprob = fused_grpo_loss(
+        hidden, case.lm_head.to(gpu), case.tokens.to(gpu), case.logprobs.to(gpu),
+        case.advantages.to(gpu), case.assistant_mask.to(gpu), case.weights.to(gpu))
+    loss.backward()
+    assert (logprob.cpu() - ref["logprobs"]).abs().max().item() <= 2e-3 * 25
+    assert abs(loss.item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item()) + 2e-6
+    assert torch.isfinite(hidden.grad).all()
+    assert rel_l2(hidden.grad.float().cpu(), ref["d_hidden"]) <= GRAD_TOL
+
+
+def test_fused_target_88_nats_under_the_maximum_is_loud(artk_lib, gpu):
+    """A sampled token whose logit lies more than 88 nats under its row's largest one (probability
+    below e^-88: it cannot have been sampled) overflows the exponential stash: that row's d_hidden is
+    not finite, every other row is unaffected."""
+    T, H, V = 256, 64, 1024
+    hidden = torch.zeros(1, T, H, dtype=torch.bfloat16)
+    hidden[0, :, 0] = 1.0
+    lm_head = torch.zeros(V, H, dtype=torch.bfloat16)
+    lm_head[:, 0] = -20.0
+    lm_head[7, 0] = 50.0                      # one dominant logit
+    lm_head[9, 0] = -45.0                     # 95 nats under it
+    lm_head[:, 1] = (torch.arange(V) % 5).to(torch.bfloat16)   # (unused direction: hidden[.., 1] = 0)
+    tokens = torch.full((1, T), 7, dtype=torch.int64)
+    tokens[0, 101] = 9                        # position 100's target
+    old = torch.zeros(1, T)
+    old[0, 101] = -95.0                       # ratio 1: the row has a non-zero coefficient
+    adv = torch.ones(1, T)
+    mask = torch.ones(1, T, dtype=torch.bool)
+    w = torch.ones(1, T)
+    h = hidden.to(gpu).requires_grad_(True)
+    loss, metrics, logprob = fused_grpo_loss(h, lm_head.to(gpu), tokens.to(gpu), old.to(gpu), adv.to(gpu),
+                                             mask.to(gpu), w.to(gpu))
+    loss.backward()
+    g = h.grad[0].float().cpu()
+    assert abs(logprob[0, 100].item() + 95.0) < 1e-3
+    assert not torch.isfinite(g[100]).all()
+    others = torch.cat([g[:100], g[101:]])
+    assert torch.isfinite(others).all()
+
+
 def test_unfused_autograd_matches_oracle(artk_lib, gpu):
     """_calculate_logprobs + grpo_loss composed through torch autograd (the
     reference's call structure) against the oracle, with KL."""
