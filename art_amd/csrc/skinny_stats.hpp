@@ -73,33 +73,6 @@ __device__ __forceinline__ bf16x8 st_tr_frag(const char* tile, int lane, int k0,
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// One LDS DMA instruction (64 lanes x 16 bytes land at lds_addr + 16 lane) issued from inline
-// assembly.  Issued through the builtin, the compiler would know that LDS is being written
-// behind its back and put s_waitcnt vmcnt(0) in front of every later LDS read, which drains
-// the whole ring each tile; here the completion is tracked by hand (s_waitcnt vmcnt(n) before
-// the barrier that publishes a tile), so the instruction is kept out of its sight.
-typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t st_rsrc_t;
-__device__ __forceinline__ st_rsrc_t st_make_rsrc(const void* base, uint32_t bytes) {
-  const uint64_t a = (uint64_t)base;
-  return st_rsrc_t{(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
-}
-__device__ __forceinline__ void st_dma16(st_rsrc_t rsrc, int voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(rsrc)
-               : "memory", "m0");
-}
-// The same with 4 bytes per lane (lane i lands at lds_addr + 4 i).
-__device__ __forceinline__ void st_dma4(st_rsrc_t rsrc, int voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(rsrc)
-               : "memory", "m0");
-}
-__device__ __forceinline__ uint32_t st_lds_addr(const void* p) {
-  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
-}
-
 // NTE: 32-wide tiles of e (rank <= 32 NTE); NCT: 128-column tiles per chunk; NST: LDS stages.
 // All memory traffic of the main loop is LDS DMA, ordered by hand with s_waitcnt vmcnt(n)
 // (the compiler inserts no waits for it): per wave, a tile is 8 DMA instructions, the Y rows
@@ -141,20 +114,20 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
   // then addressed through the gather or by sorted position); reads past the end return zero
   const int64_t xbase = grouped ? 0 : t0;
   const int64_t left = ((grouped ? p.x_rows : p.T) - xbase) * p.C * 2;
-  const st_rsrc_t rsrc = st_make_rsrc(p.X + xbase * p.C, (uint32_t)(left < 0x7fffffff ? left : 0x7fffffff));
+  const dma_rsrc_t rsrc = dma_make_rsrc(p.X + xbase * p.C, (uint32_t)(left < 0x7fffffff ? left : 0x7fffffff));
   // (grouped form: up to the end of the expert's rows, so that the rows of a tile past that end
   // read as zero and add nothing to the COL product)
   const int64_t yleft = do_col ? (grouped ? (int64_t)rows_here : p.T - t0) * R * 4 : 0;
-  const st_rsrc_t yrsrc =
-      st_make_rsrc(do_col ? p.Y + t0 * R : nullptr, (uint32_t)(yleft < 0x7fffffff ? yleft : 0x7fffffff));
-  const uint32_t ring_addr = st_lds_addr(ring);
+  const dma_rsrc_t yrsrc =
+      dma_make_rsrc(do_col ? p.Y + t0 * R : nullptr, (uint32_t)(yleft < 0x7fffffff ? yleft : 0x7fffffff));
+  const uint32_t ring_addr = lds_addr_of(ring);
   constexpr int IDX_OFF = NST * ST_TILE_BYTES + YRAW_BYTES;
-  const st_rsrc_t irsrc = st_make_rsrc(GATHER ? p.gather + t0 : nullptr, GATHER ? (uint32_t)rows_here * 4u : 0u);
+  const dma_rsrc_t irsrc = dma_make_rsrc(GATHER ? p.gather + t0 : nullptr, GATHER ? (uint32_t)rows_here * 4u : 0u);
   auto issue_idx = [&](int q) {
     const int pp = lane & 31;
     int rg = q * ST_TILE + wave * 32 + (pp & 7) * 4 + (pp >> 3);
     rg = rg < rows_here ? rg : rows_here - 1;
-    st_dma4(irsrc, rg * 4, ring_addr + IDX_OFF + (wave * IDX_SLOTS + q % IDX_SLOTS) * 256);
+    dma_load4(irsrc, rg * 4, 0, ring_addr + IDX_OFF + (wave * IDX_SLOTS + q % IDX_SLOTS) * 256);
   };
   auto issue_tile = [&](int i) {
     const int rt = i / nct, ct = i - rt * nct;
@@ -177,7 +150,7 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
       else if (grouped) xrow = t0 + rg;
       const int c = (lane & 15) ^ st_swz(row);
       const int voff = (int)(xrow * p.C * 2) + (int)((c0 + ct * ST_TILE + c * 8) * 2);
-      st_dma16(rsrc, voff, stage + instr * 1024);
+      dma_load16(rsrc, voff, 0, stage + instr * 1024);
     }
   };
   // Y rows of row tile rt: 128 R floats, contiguous in memory, land as they are (R / 8 instructions per wave)
@@ -186,7 +159,7 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
     for (int k = 0; k < ny; ++k) {
       const int instr = wave * ny + k;
       const int voff = rt * ST_TILE * R * 4 + instr * 1024 + lane * 16;
-      st_dma16(yrsrc, voff, ring_addr + NST * ST_TILE_BYTES + instr * 1024);
+      dma_load16(yrsrc, voff, 0, ring_addr + NST * ST_TILE_BYTES + instr * 1024);
     }
   };
   if constexpr (GATHER) {
