@@ -484,7 +484,7 @@ __global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __r
 // and the schedule of the d_hidden GEMM over those rows.  One block.
 //   sched[0] = n_active, [1] = token tiles, [2] = K splits, [3] = work-groups
 // Rows whose coefficient is zero (non-assistant positions, zero advantage) have
-// an exactly zero d_hidden row and are skipped by K3b and K4.
+// an exactly zero d_hidden row and are skipped by K4.
 __global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restrict__ coef,
                                                             ChunkRows rows, int HT, int ksteps,
                                                             int part_rows,

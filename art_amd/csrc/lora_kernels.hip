@@ -11,8 +11,9 @@
 // The dense products run on the shared 256x256 MFMA main loop.  The rank-r
 // products ride along as extra K = 16 MFMA steps whose operands (the low-rank
 // factors) are read straight from global memory, so y and dx are each one GEMM
-// launch.  The skinny products (x A^T, g B: reductions along a row; dA, dB:
-// reductions along the token axis) are bandwidth-bound helpers.
+// launch.  The skinny products are bandwidth-bound: x A^T in the forward is a row
+// product (rowdot16_kernel); in the backward g B and dB come from one pass over g
+// and dA from one pass over x (lora_stats_kernel, skinny_stats.hpp).
 #include "common.hpp"
 #include "gemm_nt.hpp"
 #include "lora_common.hpp"
@@ -175,96 +176,6 @@ __global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restric
   }
 }
 
-// ----------------------------------------------------------------------------
-// Column products over a slab of rows, two jobs per launch (dA and dB):
-//   partial[slab][c][r] = sum_{t in slab} X[t,c] Y[t,r]     r in [r0, r0+8)
-// X [T,C] bf16, Y [T,R] f32.  A thread owns 2 columns; Y rows are staged in LDS
-// and read as broadcasts.
-// ----------------------------------------------------------------------------
-constexpr int COLDOT_MAX_ROWS = 256;
-
-struct ColdotJob {
-  const uint16_t* X;
-  const float* Y;
-  float* partial;
-  float* out;
-  int64_t C;
-  int rows_per_slab, nslab, col_blocks, transpose_out;
-};
-
-__global__ __launch_bounds__(256) void coldot8_kernel(ColdotJob a, ColdotJob b, int64_t T, int R) {
-  __shared__ float ys[COLDOT_MAX_ROWS][8];
-  const int na = a.col_blocks * a.nslab;
-  const bool first = (int)blockIdx.x < na;
-  const ColdotJob j = first ? a : b;
-  const int bid = first ? blockIdx.x : blockIdx.x - na;
-  const int slab = bid / j.col_blocks, cb = bid - slab * j.col_blocks;
-  const int64_t c = ((int64_t)cb * 256 + threadIdx.x) * 2;
-  const int r0 = blockIdx.y * 8;
-  const int64_t t0 = (int64_t)slab * j.rows_per_slab;
-  const int nrows = (int)((T - t0) < j.rows_per_slab ? (T - t0) : j.rows_per_slab);
-  for (int i = threadIdx.x; i < j.rows_per_slab * 8; i += 256) {
-    int rr = i >> 3, e = i & 7;
-    ys[rr][e] = rr < nrows ? j.Y[(t0 + rr) * R + r0 + e] : 0.f;
-  }
-  __syncthreads();
-  if (c >= j.C) return;
-  float acc[2][8];
-#pragma unroll
-  for (int q = 0; q < 2; ++q)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[q][e] = 0.f;
-  const uint16_t* xp = j.X + t0 * j.C + c;
-#pragma unroll 8
-  for (int rr = 0; rr < nrows; ++rr) {
-    float x0, x1;
-    unpack2(*(const uint32_t*)(xp + (int64_t)rr * j.C), x0, x1);
-    const floatx4 ya = *(const floatx4*)&ys[rr][0];
-    const floatx4 yb = *(const floatx4*)&ys[rr][4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      acc[0][e] += x0 * ya[e];
-      acc[1][e] += x1 * ya[e];
-      acc[0][4 + e] += x0 * yb[e];
-      acc[1][4 + e] += x1 * yb[e];
-    }
-  }
-  float* pp = j.partial + ((int64_t)slab * j.C + c) * R + r0;
-#pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    *(floatx4*)(pp + (int64_t)q * R) = floatx4{acc[q][0], acc[q][1], acc[q][2], acc[q][3]};
-    *(floatx4*)(pp + (int64_t)q * R + 4) = floatx4{acc[q][4], acc[q][5], acc[q][6], acc[q][7]};
-  }
-}
-
-// out = scale * sum over slabs (fixed order); out is [C,R], or [R,C] when
-// transpose_out.  64 outputs per block, 4 threads per output.
-__global__ __launch_bounds__(256) void coldot_reduce_kernel(ColdotJob a, ColdotJob b, int R, float scale) {
-  __shared__ float red[4][64];
-  const int nba = (int)((a.C * R + 63) / 64);
-  const bool first = (int)blockIdx.x < nba;
-  const ColdotJob j = first ? a : b;
-  const int bid = first ? blockIdx.x : blockIdx.x - nba;
-  const int64_t n = j.C * R;
-  const int64_t i = (int64_t)bid * 64 + (threadIdx.x & 63);
-  const int part = threadIdx.x >> 6;
-  float s = 0.f;
-  if (i < n)
-    for (int k = part; k < j.nslab; k += 4) s += j.partial[(int64_t)k * n + i];
-  red[part][threadIdx.x & 63] = s;
-  __syncthreads();
-  if (part == 0 && i < n) {
-    s = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x])) * scale;
-    if (j.transpose_out) {
-      const int64_t c = i / R;
-      const int r = (int)(i - c * R);
-      j.out[(int64_t)r * j.C + c] = s;
-    } else {
-      j.out[i] = s;
-    }
-  }
-}
-
 static int32_t check_lora(int64_t T, int64_t in, int64_t out, int r) {
   ARTK_CHECK_ARG(T > 0 && in > 0 && out > 0 && r > 0, "T, in, out, r must be positive");
   if (in % BK != 0 || out % BK != 0) {
@@ -317,35 +228,6 @@ static int32_t launch_rowdot(const void* X, const void* Mt, int64_t T, int64_t K
                                         out_f32, out_bf16);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
-}
-
-// Slab height for a column product over T rows of a [T,C] matrix: enough blocks
-// to fill the chip without inflating the partial buffer.
-static int coldot_rows(int64_t T, int64_t C) {
-  const int64_t col_blocks = (C / 2 + 255) / 256;
-  for (int rows : {256, 128, 64})
-    if (col_blocks * ((T + rows - 1) / rows) >= 1024) return rows;
-  return 64;
-}
-
-static ColdotJob make_job(const void* X, const float* Y, float* partial, float* out, int64_t T,
-                          int64_t C, int transpose_out) {
-  ColdotJob j;
-  j.X = (const uint16_t*)X;
-  j.Y = Y;
-  j.partial = partial;
-  j.out = out;
-  j.C = C;
-  j.rows_per_slab = coldot_rows(T, C);
-  j.nslab = (int)((T + j.rows_per_slab - 1) / j.rows_per_slab);
-  j.col_blocks = (int)((C / 2 + 255) / 256);
-  j.transpose_out = transpose_out;
-  return j;
-}
-
-static size_t coldot_partial_floats(int64_t T, int64_t C, int R) {
-  const int rows = coldot_rows(T, C);
-  return (size_t)((T + rows - 1) / rows) * C * R;
 }
 
 }  // namespace artk
