@@ -393,96 +393,6 @@ __global__ __launch_bounds__(256) void moe_rowdot16_kernel(
   }
 }
 
-// Grouped column products over the rows of one expert:
-//   out_e[c, r] = scale * sum_{i in rows(e)} X[row(i), c] Y[i, r]    r in [r0, r0+8)
-// out is [E,C,R], or [E,R,C] when transpose_out.  A block owns 128 columns of one
-// expert: 16 column groups of 8 (one 16-byte load per row) x 16 row groups (row
-// group g takes rows g, g+16, ...), merged in a fixed order: butterflies over the
-// 4 row groups of a wave, then the 4 waves through LDS.
-__global__ __launch_bounds__(256) void moe_coldot8_kernel(
-    const uint16_t* __restrict__ X, const int* __restrict__ gather, const float* __restrict__ Y,
-    const int* __restrict__ offsets, int64_t C, int R, float scale, int transpose_out,
-    float* __restrict__ out) {
-  __shared__ float ys[128][8];
-  __shared__ int rows[128];
-  __shared__ float red[3][16][65];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int cg = threadIdx.x & 15, rg = threadIdx.x >> 4;
-  const int64_t c = ((int64_t)blockIdx.x * 16 + cg) * 8;
-  const int e = blockIdx.y;
-  const int r0 = blockIdx.z * 8;
-  const int64_t begin = offsets[e], end = offsets[e + 1];
-  float acc[8][8];  // [column][r]
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-#pragma unroll
-    for (int q = 0; q < 8; ++q) acc[j][q] = 0.f;
-  for (int64_t s0 = begin; s0 < end; s0 += 128) {
-    const int nrows = (int)(end - s0 < 128 ? end - s0 : 128);
-    __syncthreads();
-    for (int i = threadIdx.x; i < 128 * 8; i += 256) {
-      const int rr = i >> 3, q = i & 7;
-      ys[rr][q] = rr < nrows ? Y[(s0 + rr) * R + r0 + q] : 0.f;
-    }
-    if (threadIdx.x < 128) {
-      const int64_t i = s0 + threadIdx.x;
-      rows[threadIdx.x] = (int)threadIdx.x < nrows ? (gather ? gather[i] : (int)i) : 0;
-    }
-    __syncthreads();
-    if (c < C) {
-#pragma unroll 4
-      for (int rr = rg; rr < nrows; rr += 16) {
-        const uint4 xv = *(const uint4*)(X + (int64_t)rows[rr] * C + c);
-        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
-        const floatx4 ya = *(const floatx4*)&ys[rr][0];
-        const floatx4 yb = *(const floatx4*)&ys[rr][4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float x0, x1;
-          unpack2(xw[j], x0, x1);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            acc[2 * j][q] += x0 * ya[q];
-            acc[2 * j + 1][q] += x1 * ya[q];
-            acc[2 * j][4 + q] += x0 * yb[q];
-            acc[2 * j + 1][4 + q] += x1 * yb[q];
-          }
-        }
-      }
-    }
-  }
-  // the 4 row groups of a wave sit 16 lanes apart
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      float v = acc[j][q];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
-      acc[j][q] = v;
-    }
-  if (wave > 0 && lane < 16) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-#pragma unroll
-      for (int q = 0; q < 8; ++q) red[wave - 1][cg][j * 8 + q] = acc[j][q];
-  }
-  __syncthreads();
-  if (wave != 0 || lane >= 16 || c >= C) return;
-  float* oe = out + (int64_t)e * C * R;
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const float v =
-          (acc[j][q] + red[0][cg][j * 8 + q] + red[1][cg][j * 8 + q] + red[2][cg][j * 8 + q]) * scale;
-      if (transpose_out)
-        oe[(int64_t)(r0 + q) * C + c + j] = v;
-      else
-        oe[(c + j) * R + r0 + q] = v;
-    }
-}
-
 __global__ __launch_bounds__(256) void transpose_bf16_batched_kernel(const uint16_t* __restrict__ in,
                                                                      uint16_t* __restrict__ out,
                                                                      int64_t R, int64_t C) {
@@ -561,16 +471,6 @@ static int32_t launch_moe_rowdot(const void* X, const int* gather, const uint16_
   dim3 grid((unsigned)((n_rows + 15) / 16 + E), (unsigned)(RP / 16));
   moe_rowdot16_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, gather, Mt, offsets, blk_prefix, E, K,
                                             R, RP, scale, out_f32, out_bf16);
-  ARTK_CHECK_LAUNCH();
-  return ARTK_OK;
-}
-
-static int32_t launch_moe_coldot(const void* X, const int* gather, const float* Y, const int* offsets,
-                                 int E, int64_t C, int R, float scale, int transpose_out, float* out,
-                                 hipStream_t st) {
-  dim3 grid((unsigned)((C / 2 + 63) / 64), (unsigned)E, (unsigned)(R / 8));
-  moe_coldot8_kernel<<<grid, 256, 0, st>>>((const uint16_t*)X, gather, Y, offsets, C, R, scale,
-                                           transpose_out, out);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -730,13 +630,9 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
   if ((rc = launch_moe_gemm(W_t, g, nullptr, c.At, c.gb16, dx, expert_offsets, tile_prefix, n_rows, in, out,
                             E, r, RP, st)))
     return rc;
-  // one pass over x: dA_e [r,in] = s (g B_e)^T x.  (With a row gather the last tile of a row may
-  // reach past the row: only taken when the rows are whole tiles wide, so nothing is read
-  // beyond the last row of x, whose count this call does not know.)
-  if (gather == nullptr || in % ST_TILE == 0)
-    return launch_stats_grouped(x, gather ? (int64_t)0x3fffffff / in : n_rows, gather, n_rows, in, nullptr, c.gb,
-                                r, E, expert_offsets, nullptr, dA, scale, 1, c.dummy, st);
-  return launch_moe_coldot(x, gather, c.gb, expert_offsets, E, in, r, scale, 1, dA, st);
+  // one pass over x (through the row gather when there is one): dA_e [r,in] = s (g B_e)^T x
+  return launch_stats_grouped(x, gather ? (int64_t)0x3fffffff / in : n_rows, gather, n_rows, in, nullptr, c.gb, r,
+                              E, expert_offsets, nullptr, dA, scale, 1, c.dummy, st);
 }
 
 int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_t R, int64_t C,

@@ -149,7 +149,12 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
       if constexpr (GATHER) xrow = gidx[k];
       else if (grouped) xrow = t0 + rg;
       const int c = (lane & 15) ^ st_swz(row);
-      const int voff = (int)(xrow * p.C * 2) + (int)((c0 + ct * ST_TILE + c * 8) * 2);
+      // columns past the end of a row (the ragged last column tile) re-read the row's first
+      // chunk instead: their ROW factor is zero and their COL results are never stored, and
+      // nothing is read outside the row, whatever follows it in memory
+      int64_t col = c0 + ct * ST_TILE + c * 8;
+      col = col < p.C ? col : 0;
+      const int voff = (int)(xrow * p.C * 2) + (int)(col * 2);
       dma_load16(rsrc, voff, 0, stage + instr * 1024);
     }
   };
