@@ -110,6 +110,33 @@ def test_grouped_lora_matches_oracle(artk_lib, gpu, T, H, I, E, k, use_gather):
     assert rel_l2(dB.cpu(), dB0) <= TOL
 
 
+@pytest.mark.parametrize("r,use_gather", [(40, True), (64, False), (16, True)])
+def test_grouped_lora_ranks(artk_lib, gpu, r, use_gather):
+    """Ranks other than 8: above 32 the one-pass backward runs its two-tile-per-rank shape (256-column
+    chunks, two stages), with and without the row gather."""
+    print(f"moe grouped rank {r} gather={use_gather}", flush=True)
+    T, H, I, E, k = 384, 320, 192, 8, 2
+    g = torch.Generator().manual_seed(100 + r)
+    logits = torch.randn(T, E, generator=g)
+    rt, ref = check_routing(logits, k, gpu)
+    n_rows = T * k
+    x = torch.randn(T if use_gather else n_rows, H, generator=g).to(torch.bfloat16)
+    W, A, B = make_experts(E, I, H, r, 11)
+    up = torch.randn(n_rows, I, generator=g).to(torch.bfloat16)
+    y0, dx0, dA0, dB0 = moe_oracle.grouped_lora_grads(
+        x, ref["row_token"] if use_gather else None, W, A, B, 0.5, ref["offsets"], up)
+    gather = rt.row_token if use_gather else None
+    y, xa = ops.moe_lora_grouped_fwd(x.to(gpu), gather, W.to(gpu), A.to(gpu), B.to(gpu), 0.5, rt)
+    dx, dA, dB = ops.moe_lora_grouped_bwd(up.to(gpu), x.to(gpu), gather, ops.transpose_batched(W.to(gpu)),
+                                          A.to(gpu), B.to(gpu), xa, 0.5, rt)
+    assert rel_l2(y.cpu().float(), y0) <= TOL
+    if use_gather:
+        dx = dx[rt.inv_perm.long()].view(T, k, H).float().sum(1)
+    assert rel_l2(dx.cpu().float(), dx0) <= TOL
+    assert rel_l2(dA.cpu(), dA0) <= TOL
+    assert rel_l2(dB.cpu(), dB0) <= TOL
+
+
 @pytest.mark.parametrize("use_gather", [True, False])
 def test_grouped_lora_with_empty_experts(artk_lib, gpu, use_gather):
     """Experts that no token chose: their dA_e and dB_e are exactly zero, the others match the oracle
