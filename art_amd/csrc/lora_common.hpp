@@ -86,8 +86,10 @@ __device__ __forceinline__ void unpack2(uint32_t w, float& lo, float& hi) {
   hi = __uint_as_float(w & 0xffff0000u);
 }
 
-// dst[c, r] = src[r, c] for small bf16 matrices; `which` selects one of two jobs so
-// that both transposes of a LoRA backward share a launch.
+// dst[c, r] = src[r, c] for n bf16 matrices [R, C] with R and C multiples of 8 (LoRA factors: one
+// dimension is the rank); blockIdx.y selects one of two jobs so that both transposes of a LoRA
+// backward share a launch.  A thread turns an 8 x 8 block in registers: eight 16-byte loads along
+// the rows of src, eight 16-byte stores along the rows of dst.
 struct SmallTranspose {
   const uint16_t* src;
   uint16_t* dst;
@@ -95,11 +97,33 @@ struct SmallTranspose {
 };
 __global__ __launch_bounds__(256) static void small_transpose2_kernel(SmallTranspose a, SmallTranspose b) {
   const SmallTranspose t = blockIdx.y == 0 ? a : b;
+  const int64_t RB = t.R / 8, CB = t.C / 8;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= t.n * t.R * t.C) return;
-  const int64_t m = i / (t.R * t.C), j = i - m * t.R * t.C;
-  const int64_t c = j / t.R, r = j - c * t.R;  // dst index [c][r]
-  t.dst[i] = t.src[m * t.R * t.C + r * t.C + c];
+  if (i >= t.n * RB * CB) return;
+  const int64_t m = i / (RB * CB), j = i - m * RB * CB;
+  const int64_t rb = j / CB, cb = j - rb * CB;
+  const uint16_t* src = t.src + m * t.R * t.C + rb * 8 * t.C + cb * 8;
+  uint16_t* dst = t.dst + m * t.R * t.C + cb * 8 * t.R + rb * 8;
+  uint32_t in[8][4];  // in[r][k]: columns 2k, 2k + 1 of row r
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const uint4 v = *(const uint4*)(src + r * t.C);
+    in[r][0] = v.x;
+    in[r][1] = v.y;
+    in[r][2] = v.z;
+    in[r][3] = v.w;
+  }
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = (in[2 * k][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+      const uint32_t hi = (in[2 * k + 1][c >> 1] >> (16 * (c & 1))) & 0xffffu;
+      o[k] = lo | (hi << 16);
+    }
+    *(uint4*)(dst + c * t.R) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
 }
 
 static inline int32_t launch_small_transpose2(const void* s0, void* d0, int64_t n0, int64_t R0, int64_t C0,
@@ -107,7 +131,7 @@ static inline int32_t launch_small_transpose2(const void* s0, void* d0, int64_t 
                                               hipStream_t st) {
   SmallTranspose a{(const uint16_t*)s0, (uint16_t*)d0, n0, R0, C0};
   SmallTranspose b{(const uint16_t*)s1, (uint16_t*)d1, n1, R1, C1};
-  const int64_t big = n0 * R0 * C0 > n1 * R1 * C1 ? n0 * R0 * C0 : n1 * R1 * C1;
+  const int64_t big = (n0 * R0 * C0 > n1 * R1 * C1 ? n0 * R0 * C0 : n1 * R1 * C1) / 64;  // 8 x 8 blocks
   dim3 grid((unsigned)((big + 255) / 256), 2);
   small_transpose2_kernel<<<grid, 256, 0, st>>>(a, b);
   ARTK_CHECK_LAUNCH();

@@ -298,7 +298,7 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
   int32_t rc = check_lora(T, in, out, r);
   if (rc) return rc;
   ARTK_CHECK_ARG(g && x && W_t && A && B && xa && dx && dA && dB, "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(dx) && aligned16(xa) &&
+  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(A) && aligned16(B) && aligned16(dx) && aligned16(xa) &&
                      aligned16(dA) && aligned16(dB),
                  "pointers must be 16-byte aligned");
   const int RP = round16(r);

@@ -600,7 +600,7 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
   ARTK_CHECK_ARG(g && x && W_t && A && B && xa && expert_offsets && tile_prefix && blk_prefix && dx &&
                      dA && dB,
                  "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(dx) && aligned16(xa) &&
+  ARTK_CHECK_ARG(aligned16(g) && aligned16(x) && aligned16(W_t) && aligned16(A) && aligned16(B) && aligned16(dx) && aligned16(xa) &&
                      aligned16(dA) && aligned16(dB),
                  "pointers must be 16-byte aligned");
   if (n_rows * (in > out ? in : out) * 2 >= (1ll << 31)) {
