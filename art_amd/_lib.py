@@ -76,6 +76,7 @@ SIGNATURES = {
     "artk_profile_enable": (_i32, [_i32]),
     "artk_profile_collect": (_i32, [_i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "artk_mfma_loop": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
+    "artk_mfma_loop16": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
     "artk_stream_copy": (_i32, [_p, _p, _i64, _p]),
 }
 

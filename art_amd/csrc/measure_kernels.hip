@@ -41,6 +41,48 @@ __global__ __launch_bounds__(512) void mfma_loop_kernel(const uint16_t* __restri
   sink[gid] = s;
 }
 
+// The same amount of matrix work per round on MFMA 16x16x32 (8 x 4 tiles of 16 x 16 per
+// wave, the same 128 accumulators): this shape moves a quarter of the accumulator data
+// per instruction for half the flops, and sustains a higher rate under the power limit.
+__global__ __launch_bounds__(512) void mfma_loop16_kernel(const uint16_t* __restrict__ operands,
+                                                          int64_t n_operands, int64_t iters,
+                                                          float* __restrict__ sink) {
+  const int64_t gid = (int64_t)blockIdx.x * 512 + threadIdx.x;
+  bf16x8 a[2][8], b[2][4];  // the two K = 32 steps of one 64-wide K stage
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[s][i] = *(const bf16x8*)(operands + ((gid * 24 + s * 12 + i) * 8) % (n_operands - 8));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      b[s][i] = *(const bf16x8*)(operands + ((gid * 24 + s * 12 + 8 + i) * 8) % (n_operands - 8));
+  }
+  floatx4 c[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c[i][j][e] = 0.f;
+  for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], c[i][j], 0, 0, 0);
+  }
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) t += c[i][j][e];
+  sink[gid] = t;
+}
+
 __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ src,
                                                           uint4* __restrict__ dst, int64_t n16) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256)
@@ -61,6 +103,18 @@ int32_t artk_mfma_loop(const void* operands, int64_t n_operands, int64_t iters, 
   ARTK_CHECK_ARG(iters > 0 && blocks > 0 && blocks <= 65536, "iters and blocks must be positive (blocks <= 65536)");
   mfma_loop_kernel<<<(unsigned)blocks, 512, 0, (hipStream_t)stream>>>((const uint16_t*)operands, n_operands,
                                                                       iters, sink);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_mfma_loop16(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
+                         float* sink, artk_stream_t stream) {
+  ARTK_CHECK_ARG(operands && sink, "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(operands), "operands must be 16-byte aligned");
+  ARTK_CHECK_ARG(n_operands >= 4096 && n_operands % 8 == 0, "n_operands must be a multiple of 8, at least 4096");
+  ARTK_CHECK_ARG(iters > 0 && blocks > 0 && blocks <= 65536, "iters and blocks must be positive (blocks <= 65536)");
+  mfma_loop16_kernel<<<(unsigned)blocks, 512, 0, (hipStream_t)stream>>>((const uint16_t*)operands, n_operands,
+                                                                        iters, sink);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

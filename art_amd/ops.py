@@ -657,14 +657,20 @@ def profile_collect(kind: int) -> Tuple[float, int]:
 # -----------------------------------------------------------------------------
 # ceilings of the part (measurement aids)
 # -----------------------------------------------------------------------------
-def mfma_loop(operands: torch.Tensor, iters: int, blocks: int, sink: Optional[torch.Tensor] = None) -> float:
-    """Launches the MFMA-only loop; returns the flop it executes (time it with events)."""
+def mfma_loop(operands: torch.Tensor, iters: int, blocks: int, sink: Optional[torch.Tensor] = None,
+              shape: str = "32x32x16") -> float:
+    """Launches the MFMA-only loop (``shape``: "32x32x16", the main loop's instruction, or "16x16x32");
+    returns the flop it executes (time it with events)."""
     _need(operands, "operands", torch.bfloat16)
+    if shape not in ("32x32x16", "16x16x32"):
+        raise ValueError("shape must be '32x32x16' or '16x16x32'")
     if sink is None:
         sink = torch.empty(blocks * 512, dtype=torch.float32, device=operands.device)
     _need(sink, "sink", torch.float32, (blocks * 512,))
-    _lib.check(_lib.load().artk_mfma_loop(operands.data_ptr(), operands.numel(), int(iters), int(blocks),
-                                          sink.data_ptr(), _stream(operands.device)))
+    lib = _lib.load()
+    fn = lib.artk_mfma_loop if shape == "32x32x16" else lib.artk_mfma_loop16
+    _lib.check(fn(operands.data_ptr(), operands.numel(), int(iters), int(blocks), sink.data_ptr(),
+                  _stream(operands.device)))
     return float(blocks) * 8 * iters * 32 * 32768.0
 
 

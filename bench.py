@@ -913,6 +913,7 @@ def bench_ceiling(args, hidden=None, lm_head=None, seconds=0.6):
     iters = 40000
     flop = float(blocks) * 8 * iters * 32 * 32768.0
     out["mfma_only"] = run(lambda: ops.mfma_loop(operands, iters, blocks, sink), flop=flop)
+    out["mfma_only_16x16x32"] = run(lambda: ops.mfma_loop(operands, iters, blocks, sink, shape="16x16x32"), flop=flop)
     gemm_flop = 2.0 * chunk * V * H
     w_t = lm_head.t()
     dst = torch.empty((chunk, V), dtype=torch.bfloat16, device=dev)

@@ -405,10 +405,14 @@ int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches);
  *   (bf16 [n_operands], n_operands >= 4096, a multiple of 8); no LDS, no memory
  *   traffic inside the loop.  Work: blocks * 8 * iters * 32 * 32768 flop.
  *   sink f32 [blocks * 512] receives a checksum per lane.
+ * artk_mfma_loop16: the same arguments and the same work per round as 64 MFMA
+ *   16x16x32 instructions on 8 x 4 tiles of 16 x 16 per wave.
  * artk_stream_copy: dst[i] = src[i], 16 bytes per lane and step (bytes % 16 == 0).
  * ------------------------------------------------------------------------- */
 int32_t artk_mfma_loop(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
                        float* sink, artk_stream_t stream);
+int32_t artk_mfma_loop16(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
+                         float* sink, artk_stream_t stream);
 int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_t stream);
 
 #ifdef __cplusplus

@@ -1,0 +1,71 @@
+"""The measurement aids of the library: MFMA-only loops and the plain copy.
+
+The loops have no counterpart in the reference; what is checked is that they do the matrix
+work they are credited with: the sum of a wave's accumulators after one round equals the
+closed form  sum_s sum_g (sum of the A fragments of K group g) . (sum of the B fragments of g),
+evaluated in float64 from the operand indices the kernels document.
+"""
+import numpy as np
+import pytest
+import torch
+
+from art_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def wave_sums_closed_form(operands, shape):
+    n = operands.numel()
+    x = operands.float().double().numpy()
+    if shape == "32x32x16":
+        steps, per_step, na, nb, group_shift = 4, 6, 4, 2, 5
+    else:
+        steps, per_step, na, nb, group_shift = 2, 12, 8, 4, 4
+    out = np.zeros(8)
+    gid = np.arange(512)
+
+    def frag(s, slot):  # [512 lanes, 8]
+        base = ((gid * 24 + s * per_step + slot) * 8) % (n - 8)
+        return x[base[:, None] + np.arange(8)[None, :]]
+
+    for s in range(steps):
+        a = sum(frag(s, i) for i in range(na))
+        b = sum(frag(s, na + j) for j in range(nb))
+        for wave in range(8):
+            for g in range(64 >> group_shift):
+                lanes = [wave * 64 + l for l in range(64) if (l >> group_shift) == g]
+                out[wave] += float(a[lanes].sum(0) @ b[lanes].sum(0))
+    return out
+
+
+@pytest.mark.parametrize("shape", ["32x32x16", "16x16x32"])
+def test_mfma_loop_does_the_work_it_is_credited_with(artk_lib, gpu, shape):
+    print(f"mfma_loop {shape}", flush=True)
+    g = torch.Generator().manual_seed(11)
+    operands = torch.randn(1 << 14, generator=g).to(torch.bfloat16)
+    sink = torch.zeros(512, dtype=torch.float32, device=gpu)
+    flop = ops.mfma_loop(operands.to(gpu), 1, 1, sink, shape=shape)
+    assert flop == 8 * 32 * 32768.0
+    got = sink.cpu().double().view(8, 64).sum(1).numpy()
+    want = wave_sums_closed_form(operands, shape)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-3 * scale + 1e-2, (got, want)
+    sink3 = torch.zeros_like(sink)
+    ops.mfma_loop(operands.to(gpu), 3, 1, sink3, shape=shape)
+    got3 = sink3.cpu().double().view(8, 64).sum(1).numpy()
+    assert np.abs(got3 - 3 * want).max() <= 3e-3 * scale + 3e-2
+
+
+def test_mfma_loop_rejects_bad_arguments(artk_lib, gpu):
+    operands = torch.zeros(4096, dtype=torch.bfloat16, device=gpu)
+    with pytest.raises(ValueError):
+        ops.mfma_loop(operands, 1, 1, shape="4x4x4")
+    with pytest.raises((ValueError, RuntimeError)):
+        ops.mfma_loop(operands[:1024], 1, 1)
+
+
+def test_stream_copy_is_a_copy(artk_lib, gpu):
+    src = torch.arange(1 << 20, dtype=torch.int32, device=gpu)
+    dst = torch.zeros_like(src)
+    assert ops.stream_copy(src, dst) == src.numel() * 4
+    assert torch.equal(src, dst)
