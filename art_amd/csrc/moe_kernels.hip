@@ -577,7 +577,7 @@ static void carve_moe_bwd(Workspace& ws, int64_t n_rows, int64_t in, int64_t out
   c.At = ws.take<uint16_t>((size_t)E * in * r);   // [E,in,r]
   c.gb = ws.take<float>((size_t)n_rows * r);
   c.gb16 = ws.take<uint16_t>((size_t)n_rows * RP);
-  c.rowp = ws.take<float>((size_t)stats_grouped_chunks(out, r) * n_rows * r);
+  c.rowp = ws.take<float>((size_t)stats_grouped_chunks(out, r, E) * n_rows * r);
   c.dummy = ws.take<float>(1024);
 }
 
@@ -623,7 +623,7 @@ int32_t artk_moe_lora_grouped_bwd(const void* g, const void* x, const int32_t* g
                                  scale, 0, c.dummy, st)))
     return rc;
   {
-    StatsReduceJob ja{c.rowp, stats_grouped_chunks(out, r), n_rows, 1.f, c.gb, 0, c.gb16, RP, scale};
+    StatsReduceJob ja{c.rowp, stats_grouped_chunks(out, r, E), n_rows, 1.f, c.gb, 0, c.gb16, RP, scale};
     StatsReduceJob jb{nullptr, 0, 0, 0.f, nullptr, 0, nullptr, 0, 0.f};
     if ((rc = launch_stats_reduce(ja, jb, r, st))) return rc;
   }

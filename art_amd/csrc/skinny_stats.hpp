@@ -37,6 +37,7 @@ struct StatsParams {
   float* col_part;    // [n_slabs][C][R]
   float* row_dummy;   // 1024 floats that out-of-range lanes of a ROW flush write to
   int R, rows_per_slab, n_slabs, n_chunks;
+  int cc;  // columns per chunk: a multiple of 128, at most the kernel's NCT * 128
   // Grouped form (offsets != nullptr): slab s is the run of rows offsets[s] .. offsets[s+1] of
   // expert s, F is [n_slabs,R,C], row i reads X row gather[i] (gather may be null), and the
   // COL product of a slab is complete: col_scale times it goes straight to col_out
@@ -99,11 +100,11 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
   const int slab = blockIdx.x / p.n_chunks, chunk = blockIdx.x - slab * p.n_chunks;
   const bool grouped = p.offsets != nullptr;
   const int64_t t0 = grouped ? (int64_t)p.offsets[slab] : (int64_t)slab * p.rows_per_slab;
-  const int64_t c0 = (int64_t)chunk * CC;
+  const int64_t c0 = (int64_t)chunk * p.cc;
   const int rows_here = grouped ? p.offsets[slab + 1] - p.offsets[slab]
                                 : (int)(p.T - t0 < p.rows_per_slab ? p.T - t0 : p.rows_per_slab);
   const int n_rt = (rows_here + ST_TILE - 1) / ST_TILE;
-  const int cols_here = (int)(p.C - c0 < CC ? p.C - c0 : CC);
+  const int cols_here = (int)(p.C - c0 < p.cc ? p.C - c0 : p.cc);
   const int nct = (cols_here + ST_TILE - 1) / ST_TILE;
   const int nt = n_rt * nct;
   const bool do_row = p.F != nullptr, do_col = p.Y != nullptr;
@@ -375,19 +376,40 @@ static inline int stats_num_cus() {
 // Chunk width by rank (the factor and the accumulators of a chunk live in LDS / registers);
 // slab height so that the grid is one round of work-groups (one fits per CU) when the matrix
 // is large enough: a second, partly filled round would cost as much as the first.
+// Cost of a grid in half tile times: rounds of work-groups on the CUs, each as long as its tiles
+// (a row tile of cct column tiles also writes its ROW partial, about half a tile time) plus
+// about two tile times of set-up (factor load, filling the ring, flushing the accumulators).
+static inline int64_t stats_grid_cost(int64_t blocks, int64_t row_tiles_per_block, int cct) {
+  const int64_t cus = stats_num_cus();
+  return ((blocks + cus - 1) / cus) * (row_tiles_per_block * (2 * cct + 1) + 4);
+}
+
 static inline StatsGeom stats_geom(int64_t T, int64_t C, int r) {
-  StatsGeom g;
-  g.cc = r > 32 ? 256 : 512;
-  g.n_chunks = (int)((C + g.cc - 1) / g.cc);
-  const int64_t row_tiles = (T + ST_TILE - 1) / ST_TILE;
-  int64_t want = stats_num_cus() / g.n_chunks;
-  want = want < 1 ? 1 : (want > row_tiles ? row_tiles : want);
-  g.rows_per_slab = (int)((row_tiles + want - 1) / want) * ST_TILE;
+  const int max_cct = r > 32 ? 2 : 4;  // column tiles per chunk the kernel holds accumulators for
+  const int64_t row_tiles = (T + ST_TILE - 1) / ST_TILE, col_tiles = (C + ST_TILE - 1) / ST_TILE;
   // row offsets inside a slab are 31-bit byte offsets
-  const int64_t cap = ((1ll << 31) - 1) / (2 * C) / ST_TILE * ST_TILE;
-  if (g.rows_per_slab > cap) g.rows_per_slab = (int)(cap < ST_TILE ? ST_TILE : cap);
-  g.n_slabs = (int)((T + g.rows_per_slab - 1) / g.rows_per_slab);
-  return g;
+  const int64_t cap = ((1ll << 31) - 1) / (2 * C) / ST_TILE;
+  StatsGeom best{};
+  int64_t best_cost = -1;
+  for (int cct = max_cct; cct >= 1; --cct) {
+    const int64_t n_chunks = (col_tiles + cct - 1) / cct;
+    int64_t want = stats_num_cus() / n_chunks;
+    want = want < 1 ? 1 : (want > row_tiles ? row_tiles : want);
+    for (int64_t w = want; w <= want + 1 && w <= row_tiles; ++w) {
+      int64_t slab_tiles = (row_tiles + w - 1) / w;
+      if (slab_tiles > cap) slab_tiles = cap < 1 ? 1 : cap;
+      const int64_t n_slabs = (row_tiles + slab_tiles - 1) / slab_tiles;
+      const int64_t cost = stats_grid_cost(n_slabs * n_chunks, slab_tiles, cct);
+      if (best_cost < 0 || cost < best_cost) {
+        best_cost = cost;
+        best.cc = cct * ST_TILE;
+        best.n_chunks = (int)n_chunks;
+        best.rows_per_slab = (int)(slab_tiles * ST_TILE);
+        best.n_slabs = (int)n_slabs;
+      }
+    }
+  }
+  return best;
 }
 
 static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const uint16_t* F, const float* Y, int r,
@@ -412,6 +434,7 @@ static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const ui
   p.rows_per_slab = g.rows_per_slab;
   p.n_slabs = g.n_slabs;
   p.n_chunks = g.n_chunks;
+  p.cc = g.cc;
   const unsigned grid = (unsigned)(g.n_slabs * g.n_chunks);
   if (r > 32)
     lora_stats_kernel<2, 2, 2, false><<<grid, 256, 0, st>>>(p);
@@ -424,8 +447,23 @@ static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const ui
 
 // Grouped form: slab = expert.  ROW partials go to row_part [n_chunks][n_rows][r]; the COL
 // product of each expert is written to col_out, scaled.
-static inline int stats_grouped_chunks(int64_t C, int r) {
-  const int cc = r > 32 ? 256 : 512;
+static inline int stats_grouped_cc(int64_t C, int r, int E) {
+  const int max_cct = r > 32 ? 2 : 4;
+  const int64_t col_tiles = (C + ST_TILE - 1) / ST_TILE;
+  int best = max_cct;
+  int64_t best_cost = -1;
+  for (int cct = max_cct; cct >= 1; --cct) {
+    const int64_t n_chunks = (col_tiles + cct - 1) / cct;
+    const int64_t cost = stats_grid_cost((int64_t)E * n_chunks, 2, cct);  // a couple of row tiles per expert
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = cct;
+    }
+  }
+  return best * ST_TILE;
+}
+static inline int stats_grouped_chunks(int64_t C, int r, int E) {
+  const int cc = stats_grouped_cc(C, r, E);
   return (int)((C + cc - 1) / cc);
 }
 static inline int32_t launch_stats_grouped(const void* X, int64_t x_rows, const int* gather, int64_t n_rows,
@@ -451,7 +489,8 @@ static inline int32_t launch_stats_grouped(const void* X, int64_t x_rows, const 
   p.R = r;
   p.rows_per_slab = 0;
   p.n_slabs = E;
-  p.n_chunks = stats_grouped_chunks(C, r);
+  p.cc = stats_grouped_cc(C, r, E);
+  p.n_chunks = stats_grouped_chunks(C, r, E);
   const unsigned grid = (unsigned)(E * p.n_chunks);
   if (gather) {
     if (r > 32)
