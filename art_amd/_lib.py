@@ -78,8 +78,15 @@ SIGNATURES = {
     "artk_mfma_loop": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
     "artk_mfma_loop16": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
     "artk_stream_copy": (_i32, [_p, _p, _i64, _p]),
+    "artk_lds_probe": (_i32, [_i32, _i32, _i32, _p, _i64, _i32, _p, _p]),
 }
 
+
+
+class LoraProjStruct(C.Structure):
+    """artk_lora_proj_t of include/artk.h."""
+    _fields_ = [("W", _p), ("W_t", _p), ("A", _p), ("B", _p), ("bias", _p), ("y", _p), ("g", _p), ("xa", _p),
+                ("dA", _p), ("dB", _p), ("out", _i64), ("r", _i32)]
 
 
 class Nf4Struct(C.Structure):
@@ -96,6 +103,10 @@ SIGNATURES.update({
     "artk_lora_linear_fwd_nf4": (
         _i32, [_p, C.POINTER(Nf4Struct), _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
     "artk_lora_linear_bwd_nf4_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "artk_lora_linear_multi_fwd_workspace_bytes": (_sz, [_i64, _i64, C.POINTER(LoraProjStruct), _i32]),
+    "artk_lora_linear_multi_fwd": (_i32, [_p, C.POINTER(LoraProjStruct), _i32, _f32, _i64, _i64, _p, _sz, _p]),
+    "artk_lora_linear_multi_bwd_workspace_bytes": (_sz, [_i64, _i64, C.POINTER(LoraProjStruct), _i32]),
+    "artk_lora_linear_multi_bwd": (_i32, [_p, C.POINTER(LoraProjStruct), _i32, _f32, _i64, _i64, _p, _p, _sz, _p]),
     "artk_lora_linear_bwd_nf4": (
         _i32, [_p, _p, C.POINTER(Nf4Struct), _p, _p, _p, _f32, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),
 })

@@ -79,6 +79,6 @@ int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches) 
   return ARTK_OK;
 }
 
-int32_t artk_abi_version(void) { return 3; }
+int32_t artk_abi_version(void) { return 4; }
 const char* artk_last_error(void) { return artk::g_err; }
 }

@@ -369,7 +369,7 @@ __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
 // Loss kernels
 // ----------------------------------------------------------------------------
 
-// Number of positions whose (shifted) assistant mask is set. One block.
+// count[0] = number of positions whose (shifted) assistant mask is set; count[1] = 0. One block.
 __global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restrict__ mask,
                                                           int64_t T, int64_t S, int shift,
                                                           int* __restrict__ count) {
@@ -386,7 +386,8 @@ __global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restr
   if (threadIdx.x == 0) {
     int s = 0;
     for (int i = 0; i < 16; ++i) s += red[i];
-    *count = s;
+    count[0] = s;
+    count[1] = 0;  // rows dropped by splitk_reduce_kernel (fused step only)
   }
 }
 
@@ -442,13 +443,14 @@ __global__ __launch_bounds__(256) void grpo_loss_tok_kernel(LossParams p) {
   if (p.coef) p.coef[i] = (wm != 0.f) ? g * wm / denom : 0.f;
 }
 
-// scalars = {loss, mean_policy_loss, mean_kl, mask_count}. One block; fixed
+// scalars = {loss, mean_policy_loss, mean_kl, mask_count} and, with `with_dropped` (the fused
+// step), scalars[4] = count[1], the rows whose gradient was dropped.  One block; fixed
 // summation order, so the result is bit-reproducible run to run.
 __global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __restrict__ pl_tok,
                                                                 const float* __restrict__ kl_tok,
                                                                 int64_t T,
                                                                 const int* __restrict__ count,
-                                                                float beta,
+                                                                float beta, int with_dropped,
                                                                 float* __restrict__ scalars) {
   __shared__ double red[2][16];
   double a = 0.0, b = 0.0;
@@ -476,6 +478,7 @@ __global__ __launch_bounds__(1024) void grpo_loss_reduce_kernel(const float* __r
     scalars[1] = mpl;
     scalars[2] = mkl;
     scalars[3] = (float)(*count);
+    if (with_dropped) scalars[4] = (float)count[1];
   }
 }
 
@@ -561,9 +564,9 @@ __global__ __launch_bounds__(1024) void compact_rows_kernel(const float* __restr
 // logit: softmax is invariant to the shift, the target was sampled from (nearly) this
 // distribution, so its logit is a reference within a few tens of nats of the row's maximum,
 // and bf16 has the exponent range of fp32 — exp(z - ref) is representable unless a logit
-// exceeds the target's by 88 nats, i.e. unless the sampled token has probability below
-// e^-88 under the current policy; such a row's d_hidden comes out as inf / NaN, not as a
-// silently wrong number.  With the exponentials in the stash the softmax gradient needs no
+// exceeds the target's by 88 nats; a row whose lse exceeds its reference by more than 80 nats
+// (a sampled token of probability below e^-80 under the current policy) is dropped by
+// splitk_reduce_kernel: zero gradient, counted.  With the exponentials in the stash the softmax gradient needs no
 // pass of its own: d_hidden[t] = coef_t (W[y_t] - exp(ref_t - lse_t) sum_v e[t,v] W[v]),
 // the sum being the GEMM K4 and the rest the epilogue of K5.  (A stash of logits needed a
 // 2 x [Tc_active, V] read-modify-write between K2 and K4 to turn them into gradients.)
@@ -656,10 +659,18 @@ __global__ __launch_bounds__(nthreads<BWD_NI>()) void dhidden_gemm_kernel(BwdPar
   }
 }
 
+constexpr float STASH_MAX_NATS = 80.f;
+
 // K5: d_hidden row of chunk row r: 0 for inactive rows, else
 //   bf16( coef_r * ( W[y_r] - exp(ref_r - lse_r) * G ) ),  G = sum over splits of partial[active slot of r]
 // (G = sum_v exp(z[r,v] - ref_r) W[v], see target_ref_kernel); 4 elements per thread.  `out` is
 // the whole batch's d_hidden, indexed by position.
+// A row with lse_r - ref_r above STASH_MAX_NATS (its target has probability below e^-80 under
+// the current policy) is dropped: sum_v exp(z - ref) = exp(lse - ref) bounds every stashed
+// exponential and, times max |W|, every element of G, so up to the limit all of them are finite
+// in bf16 / fp32, and beyond it they may be inf or NaN.  Such a row gets a zero gradient (what
+// the reference would compute for it is cf * (W[y] - p W) with p ~ one-hot elsewhere: a finite
+// row; dropping it keeps the step finite) and is counted in *dropped (may be null).
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
                                                             const int* __restrict__ pos,
                                                             const int* __restrict__ sched,
@@ -669,14 +680,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
                                                             const float* __restrict__ ref,
                                                             const int64_t* __restrict__ ids, int64_t S,
                                                             int shift, const uint16_t* __restrict__ W,
-                                                            uint16_t* __restrict__ out) {
+                                                            uint16_t* __restrict__ out,
+                                                            int* __restrict__ dropped) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t h4 = H / 4;
   if (i >= (int64_t)rows.n() * h4) return;
   const int64_t r = i / h4, c = i - r * h4;
   const int pr = pos[r];
   floatx4 s = {0.f, 0.f, 0.f, 0.f};
-  if (pr >= 0) {
+  const bool over = pr >= 0 && !(lse[r] - ref[r] <= STASH_MAX_NATS);  // also true for NaN
+  if (over) {
+    if (c == 0 && dropped != nullptr) atomicAdd(dropped, 1);
+  } else if (pr >= 0) {
     const int nsplit = sched[2];
     const int64_t rows_per_split = (int64_t)sched[1] * TILE;
     for (int k = 0; k < nsplit; ++k)
@@ -909,7 +924,7 @@ struct BwdScratch {
 static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head, const void* lm_head_t, const int64_t* ids,
                                 int shift, const ChunkRows& rows, int64_t S, int64_t V, int64_t H,
                                 const float* lse_chunk, const float* coef_chunk, const float* ref_chunk,
-                                const BwdScratch& sc, uint16_t* d_hidden, hipStream_t st) {
+                                const BwdScratch& sc, uint16_t* d_hidden, int* dropped, hipStream_t st) {
   const int64_t Tc = rows.cap;
   const int HT = (int)((H + TILE - 1) / TILE);
   const int TT = (int)((Tc + TILE - 1) / TILE);
@@ -935,7 +950,7 @@ static int32_t launch_bwd_chunk(uint16_t* stash, const void* lm_head, const void
   const int64_t n4 = Tc * H / 4;
   splitk_reduce_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, st>>>(
       sc.partial, sc.pos, sc.sched, rows, H, V, coef_chunk, lse_chunk, ref_chunk, ids, S, shift,
-      (const uint16_t*)lm_head, d_hidden);
+      (const uint16_t*)lm_head, d_hidden, dropped);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -1125,7 +1140,7 @@ int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm
                           nullptr, c.lse_tmp, st);
     if (rc) return rc;
     rc = launch_bwd_chunk(c.stash, lm_head, lm_head_t, ids, shift, rows, S, V, H, lse + t0, grad_logprob + t0,
-                          c.ref, c.bwd, (uint16_t*)d_hidden, st);
+                          c.ref, c.bwd, (uint16_t*)d_hidden, nullptr, st);
     if (rc) return rc;
   }
   return ARTK_OK;
@@ -1178,7 +1193,7 @@ static int32_t grpo_loss_run(const float* new_logprob, const float* old_logprob,
   p.coef = coef;
   grpo_loss_tok_kernel<<<(unsigned)((T + 255) / 256), 256, 0, st>>>(p);
   ARTK_CHECK_LAUNCH();
-  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, p.ref_lp ? beta : 0.f, scalars);
+  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(pl, kl, T, count, p.ref_lp ? beta : 0.f, 0, scalars);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -1310,10 +1325,10 @@ int32_t artk_grpo_fused(const void* hidden, const void* lm_head, const void* lm_
     grpo_loss_tok_kernel<<<(unsigned)((rows.cap + 255) / 256), 256, 0, st>>>(p);
     ARTK_CHECK_LAUNCH();
     rc = launch_bwd_chunk(c.stash, lm_head, lm_head_t, tokens, 1, rows, S, V, H, c.lse, c.coef, c.ref, c.bwd,
-                          (uint16_t*)d_hidden, st);
+                          (uint16_t*)d_hidden, c.count + 1, st);
     if (rc) return rc;
   }
-  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(c.pl, c.kl, T, c.count, ref ? beta : 0.f, scalars);
+  grpo_loss_reduce_kernel<<<1, 1024, 0, st>>>(c.pl, c.kl, T, c.count, ref ? beta : 0.f, 1, scalars);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

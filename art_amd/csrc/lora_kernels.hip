@@ -37,28 +37,35 @@ struct LoraGemmParams {
   int r, RP, MT, NT;
 };
 
-// Rank-r steps and bf16 store of one finished tile.
-__device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const LoraGemmParams& p, int mt,
-                                                   int nt) {
+// Rank-r steps of one tile: acc += sum_e Qe[col, e] Pe[row, e].
+__device__ __forceinline__ void lora_tile_lowrank(TileAcc<LORA_NI>& acc, const uint16_t* Pe, int r,
+                                                  const uint16_t* Qe, int RP, int64_t M, int64_t N, int mt,
+                                                  int nt) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave_m<LORA_NI>(wave), wn = wave_n<LORA_NI>(wave);
+  int64_t prow[4], qrow[LORA_NI];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int64_t rr = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
+    prow[i] = rr < M ? rr : M - 1;
+  }
+#pragma unroll
+  for (int i = 0; i < LORA_NI; ++i) {
+    int64_t c = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, i, lane);
+    qrow[i] = c < N ? c : N - 1;
+  }
+  lowrank_steps(acc, Pe, r, r, prow, Qe, RP, RP, qrow, RP);
+}
+
+// Optional bias and the bf16 store of one finished tile: out[col, m] (out is [N, M]).
+__device__ __forceinline__ void lora_tile_store(TileAcc<LORA_NI>& acc, const uint16_t* bias, uint16_t* out,
+                                                int64_t M, int64_t N, int mt, int nt) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave_m<LORA_NI>(wave), wn = wave_n<LORA_NI>(wave);
   const int half = lane >> 5;
-  if (p.Pe != nullptr) {
-    int64_t prow[4], qrow[LORA_NI];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int64_t r = (int64_t)mt * TILE + wm * 128 + i * 32 + (lane & 31);
-      prow[i] = r < p.M ? r : p.M - 1;
-    }
-#pragma unroll
-    for (int i = 0; i < LORA_NI; ++i) {
-      int64_t c = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, i, lane);
-      qrow[i] = c < p.N ? c : p.N - 1;
-    }
-    lowrank_steps(acc, p.Pe, p.r, p.r, prow, p.Qe, p.RP, p.RP, qrow, p.RP);
-  }
-  if (p.bias != nullptr) {
+  if (bias != nullptr) {
     // element j of tile mi is output feature m0 + (j / 4) 8 + 4 half + j % 4
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
@@ -66,8 +73,8 @@ __device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const 
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         int64_t mq = m0 + q * 8 + half * 4;
-        mq = mq + 4 <= p.M ? mq : 0;  // rows past the end are never stored
-        const bf16x4 bv = *(const bf16x4*)(p.bias + mq);
+        mq = mq + 4 <= M ? mq : 0;  // rows past the end are never stored
+        const bf16x4 bv = *(const bf16x4*)(bias + mq);
 #pragma unroll
         for (int ni = 0; ni < LORA_NI; ++ni)
 #pragma unroll
@@ -81,26 +88,33 @@ __device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const 
     // lanes l and l + 32 share the column, so they take these branches together
     // (store_block_bf16 exchanges data between them)
     const int64_t col = (int64_t)nt * TILE + acc_col<LORA_NI>(wn, ni, lane);
-    const bool col_ok = col < p.N;
+    const bool col_ok = col < N;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
       const int64_t m0 = (int64_t)mt * TILE + wm * 128 + mi * 32;
-      if (m0 >= p.M) continue;  // wave-uniform
-      if (m0 + 32 <= p.M) {
-        if (col_ok) store_block_bf16(p.out + col * p.M + m0, acc.c[mi][ni], half);
+      if (m0 >= M) continue;  // wave-uniform
+      if (m0 + 32 <= M) {
+        if (col_ok) store_block_bf16(out + col * M + m0, acc.c[mi][ni], half);
       } else {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int64_t m = m0 + q * 8 + half * 4;
-          if (m >= p.M || !col_ok) continue;
+          if (m >= M || !col_ok) continue;
           bf16x4 o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][ni][q * 4 + e];
-          *(bf16x4*)(p.out + col * p.M + m) = o;
+          *(bf16x4*)(out + col * M + m) = o;
         }
       }
     }
   }
+}
+
+// Rank-r steps and bf16 store of one finished tile.
+__device__ __forceinline__ void lora_gemm_epilogue(TileAcc<LORA_NI>& acc, const LoraGemmParams& p, int mt,
+                                                   int nt) {
+  if (p.Pe != nullptr) lora_tile_lowrank(acc, p.Pe, p.r, p.Qe, p.RP, p.M, p.N, mt, nt);
+  lora_tile_store(acc, p.bias, p.out, p.M, p.N, mt, nt);
 }
 
 // Persistent work-groups: tiles t, t + grid, ...; the first DMA stage of the next
@@ -142,20 +156,102 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemm
 }
 
 // ----------------------------------------------------------------------------
+// Several products over one column operand in ONE persistent launch.
+// A job is one output matrix out[n, m] (bf16 [N, M]); it sums one or more K segments,
+//   out[n, m] = sum_s ( sum_k Q_s[n,k] P_s[m,k] + sum_e Qe_s[n,e] Pe_s[m,e] )  (+ bias[m]).
+// Forward of projections that read the same x: one job per projection (P = W_i, Q = x), one
+// segment each.  Input gradient of the same projections: one job (dx) whose segments are the
+// projections (P = W_i^T [in, out_i], Q = g_i [T, out_i], K = out_i), so the upstream gradients
+// are never concatenated and dx is written once.  A segment switch inside a tile costs one
+// exposed first-stage fetch (the two LDS stages are busy until the segment's last K step).
+// ----------------------------------------------------------------------------
+constexpr int LORA_MAX_SEG = ARTK_LORA_MULTI_MAX;
+struct LoraSeg {
+  const void* P;       // [M,K] row operand
+  const void* Q;       // [N,K] column operand
+  const uint16_t* Pe;  // [M,r]
+  const uint16_t* Qe;  // [N,RP]
+  int64_t K;
+  int r, RP;
+};
+struct LoraJob {
+  uint16_t* out;         // [N,M]
+  const uint16_t* bias;  // [M] or nullptr
+  int64_t M;
+  int MT, tile0, seg0, nseg;
+};
+struct LoraMultiParams {
+  LoraSeg seg[LORA_MAX_SEG];
+  LoraJob job[LORA_MAX_SEG];
+  int64_t N;
+  int NT, n_jobs, n_tiles;
+};
+
+__device__ __forceinline__ void lora_multi_locate(const LoraMultiParams& p, int t, int& j, int& mt, int& nt) {
+  const int id = xcd_remap(t, p.n_tiles);
+  j = 0;
+  while (j + 1 < p.n_jobs && id >= p.job[j + 1].tile0) ++j;
+  tile_coords(id - p.job[j].tile0, p.job[j].MT, p.NT, mt, nt);
+}
+
+__global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_multi_gemm_kernel(LoraMultiParams p) {
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  int t = blockIdx.x;
+  int j, mt, nt;
+  lora_multi_locate(p, t, j, mt, nt);
+  {
+    const LoraSeg& sg = p.seg[p.job[j].seg0];
+    TileLoaders<LORA_NI> first;
+    first.init(sg.P, sg.K, (int64_t)mt * TILE, p.job[j].M, sg.Q, sg.K, (int64_t)nt * TILE, p.N, 0, (int)sg.K);
+    first.issue_first(smem);
+  }
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const bool more = t2 < p.n_tiles;
+    int j2 = 0, mt2 = 0, nt2 = 0;
+    if (more) lora_multi_locate(p, t2, j2, mt2, nt2);
+    const int64_t M = p.job[j].M;
+    const int seg0 = p.job[j].seg0, nseg = p.job[j].nseg;
+    TileAcc<LORA_NI> acc;
+    acc.zero();
+    for (int s = 0; s < nseg; ++s) {
+      const LoraSeg& sg = p.seg[seg0 + s];
+      TileLoaders<LORA_NI> cur;  // the first segment's first stage is already on the way
+      cur.init(sg.P, sg.K, (int64_t)mt * TILE, M, sg.Q, sg.K, (int64_t)nt * TILE, p.N, 0, (int)sg.K);
+      if (s > 0) cur.issue_first(smem);
+      gemm_tile_run(acc, smem, cur);
+    }
+    if (more) {
+      const LoraSeg& sg = p.seg[p.job[j2].seg0];
+      TileLoaders<LORA_NI> nxt;
+      nxt.init(sg.P, sg.K, (int64_t)mt2 * TILE, p.job[j2].M, sg.Q, sg.K, (int64_t)nt2 * TILE, p.N, 0, (int)sg.K);
+      nxt.issue_first(smem);
+    }
+    for (int s = 0; s < nseg; ++s) {
+      const LoraSeg& sg = p.seg[seg0 + s];
+      if (sg.Pe != nullptr) lora_tile_lowrank(acc, sg.Pe, sg.r, sg.Qe, sg.RP, M, p.N, mt, nt);
+    }
+    lora_tile_store(acc, p.job[j].bias, p.job[j].out, M, p.N, mt, nt);
+    if (!more) break;
+    t = t2;
+    j = j2;
+    mt = mt2;
+    nt = nt2;
+  }
+}
+
+// ----------------------------------------------------------------------------
 // Row products: out[t, j] = sum_k X[t,k] Mt[j,k], Mt [R,K].  A block owns 16 rows
 // of X and 16 rows j0..j0+15 of Mt (rows >= R read as zero); its 4 waves split K.
 // Writes f32 [T,R] (unscaled) and bf16 [T,RP] (scaled, zero padded to RP).
 // ----------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restrict__ X,
-                                                       const uint16_t* __restrict__ Mt, int64_t T,
-                                                       int64_t K, int R, int RP, float scale,
-                                                       float* __restrict__ out_f32,
-                                                       uint16_t* __restrict__ out_bf16) {
-  __shared__ floatx4 red[3][64];
+__device__ __forceinline__ void rowdot16_body(const uint16_t* __restrict__ X, const uint16_t* __restrict__ Mt,
+                                              int64_t T, int64_t K, int R, int RP, float scale,
+                                              float* __restrict__ out_f32, uint16_t* __restrict__ out_bf16,
+                                              int j0, floatx4 (*red)[64]) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int64_t t0 = (int64_t)blockIdx.x * 16;
-  const int j0 = blockIdx.y * 16;
   int64_t trow = t0 + (lane & 15);
   if (trow >= T) trow = T - 1;
   const int jm = j0 + (lane & 15);
@@ -174,6 +270,33 @@ __global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restric
       }
     }
   }
+}
+
+__global__ __launch_bounds__(256) void rowdot16_kernel(const uint16_t* __restrict__ X,
+                                                       const uint16_t* __restrict__ Mt, int64_t T,
+                                                       int64_t K, int R, int RP, float scale,
+                                                       float* __restrict__ out_f32,
+                                                       uint16_t* __restrict__ out_bf16) {
+  __shared__ floatx4 red[3][64];
+  rowdot16_body(X, Mt, T, K, R, RP, scale, out_f32, out_bf16, blockIdx.y * 16, red);
+}
+
+// The same for several factors over one X in one launch: blockIdx.y walks the 16-row groups of
+// factor 0, then of factor 1, ...; each factor has its own outputs.
+struct RowdotMulti {
+  const uint16_t* Mt[LORA_MAX_SEG];
+  float* out_f32[LORA_MAX_SEG];
+  uint16_t* out_bf16[LORA_MAX_SEG];
+  int R[LORA_MAX_SEG], RP[LORA_MAX_SEG], y0[LORA_MAX_SEG + 1];
+  int n;
+};
+__global__ __launch_bounds__(256) void rowdot16_multi_kernel(const uint16_t* __restrict__ X, RowdotMulti m,
+                                                             int64_t T, int64_t K, float scale) {
+  __shared__ floatx4 red[3][64];
+  const int by = blockIdx.y;
+  int i = 0;
+  while (i + 1 < m.n && by >= m.y0[i + 1]) ++i;
+  rowdot16_body(X, m.Mt[i], T, K, m.R[i], m.RP[i], scale, m.out_f32[i], m.out_bf16[i], (by - m.y0[i]) * 16, red);
 }
 
 static int32_t check_lora(int64_t T, int64_t in, int64_t out, int r) {
@@ -250,7 +373,8 @@ int32_t artk_lora_linear_fwd(const void* x, const void* W, const void* A, const 
   int32_t rc = check_lora(T, in, out, r);
   if (rc) return rc;
   ARTK_CHECK_ARG(x && W && A && B && y && xa, "null pointer argument");
-  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(A) && aligned16(B) && aligned16(y),
+  ARTK_CHECK_ARG(aligned16(x) && aligned16(W) && aligned16(A) && aligned16(B) && aligned16(y) &&
+                     (bias == nullptr || aligned16(bias)),
                  "pointers must be 16-byte aligned");
   const int RP = round16(r);
   Workspace ws(workspace, workspace_bytes);
@@ -328,6 +452,193 @@ int32_t artk_lora_linear_bwd(const void* g, const void* x, const void* W_t, cons
     if ((rc = launch_stats_reduce(ja, jb, r, st))) return rc;
   }
   return ARTK_OK;
+}
+
+// ---- several projections of the same input -------------------------------------------------
+static int32_t check_multi(const artk_lora_proj_t* proj, int32_t n, int64_t T, int64_t in, bool bwd) {
+  ARTK_CHECK_ARG(proj != nullptr && n >= 1 && n <= ARTK_LORA_MULTI_MAX, "1 to %d projections", ARTK_LORA_MULTI_MAX);
+  int r_total = 0;
+  for (int i = 0; i < n; ++i) {
+    const artk_lora_proj_t& q = proj[i];
+    int32_t rc = check_lora(T, in, q.out, q.r);
+    if (rc) return rc;
+    r_total += q.r;
+    if (bwd) {
+      ARTK_CHECK_ARG(q.W_t && q.A && q.B && q.g && q.xa && q.dA && q.dB, "projection %d: null pointer argument", i);
+      ARTK_CHECK_ARG(aligned16(q.W_t) && aligned16(q.A) && aligned16(q.B) && aligned16(q.g) && aligned16(q.xa) &&
+                         aligned16(q.dA) && aligned16(q.dB),
+                     "projection %d: pointers must be 16-byte aligned", i);
+    } else {
+      ARTK_CHECK_ARG(q.W && q.A && q.B && q.y && q.xa, "projection %d: null pointer argument", i);
+      ARTK_CHECK_ARG(aligned16(q.W) && aligned16(q.A) && aligned16(q.B) && aligned16(q.y) && aligned16(q.xa) &&
+                         (q.bias == nullptr || aligned16(q.bias)),
+                     "projection %d: pointers must be 16-byte aligned", i);
+    }
+  }
+  if (bwd && r_total > 64) {
+    set_error("the ranks of the projections add up to %d; at most 64 in one call", r_total);
+    return ARTK_ERR_UNSUPPORTED_SHAPE;
+  }
+  return ARTK_OK;
+}
+
+static int lora_num_cus() {
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  return cus;
+}
+
+static int32_t launch_lora_multi(const LoraMultiParams& p, hipStream_t st) {
+  prof_begin(PROF_LORA_GEMM, st);
+  const int cus = lora_num_cus();
+  lora_multi_gemm_kernel<<<(unsigned)(p.n_tiles < cus ? p.n_tiles : cus), nthreads<LORA_NI>(), 0, st>>>(p);
+  prof_end(PROF_LORA_GEMM, st);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+size_t artk_lora_linear_multi_fwd_workspace_bytes(int64_t T, int64_t in, const artk_lora_proj_t* proj,
+                                                  int32_t n) {
+  (void)in;
+  Workspace ws(nullptr, 0);
+  for (int i = 0; proj != nullptr && i < n && i < ARTK_LORA_MULTI_MAX; ++i)
+    ws.take<uint16_t>((size_t)T * round16(proj[i].r));
+  return ws.used + 256;
+}
+
+int32_t artk_lora_linear_multi_fwd(const void* x, const artk_lora_proj_t* proj, int32_t n, float scale,
+                                   int64_t T, int64_t in, void* workspace, size_t workspace_bytes,
+                                   artk_stream_t stream) {
+  int32_t rc = check_multi(proj, n, T, in, false);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(x != nullptr && aligned16(x), "x must be a 16-byte aligned pointer");
+  Workspace ws(workspace, workspace_bytes);
+  uint16_t* xa16[ARTK_LORA_MULTI_MAX];
+  for (int i = 0; i < n; ++i) xa16[i] = ws.take<uint16_t>((size_t)T * round16(proj[i].r));
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  RowdotMulti m;
+  LoraMultiParams p;
+  m.n = n;
+  int y = 0, tile = 0;
+  p.N = T;
+  p.NT = (int)((T + TILE - 1) / TILE);
+  p.n_jobs = n;
+  for (int i = 0; i < n; ++i) {
+    const artk_lora_proj_t& q = proj[i];
+    const int RP = round16(q.r);
+    m.Mt[i] = (const uint16_t*)q.A;
+    m.out_f32[i] = q.xa;
+    m.out_bf16[i] = xa16[i];
+    m.R[i] = q.r;
+    m.RP[i] = RP;
+    m.y0[i] = y;
+    y += RP / 16;
+    p.seg[i] = LoraSeg{q.W, x, (const uint16_t*)q.B, xa16[i], in, q.r, RP};
+    const int MT = (int)((q.out + TILE - 1) / TILE);
+    p.job[i] = LoraJob{(uint16_t*)q.y, (const uint16_t*)q.bias, q.out, MT, tile, i, 1};
+    tile += MT * p.NT;
+  }
+  m.y0[n] = y;
+  p.n_tiles = tile;
+  dim3 grid((unsigned)((T + 15) / 16), (unsigned)y);
+  rowdot16_multi_kernel<<<grid, 256, 0, st>>>((const uint16_t*)x, m, T, in, scale);
+  ARTK_CHECK_LAUNCH();
+  return launch_lora_multi(p, st);
+}
+
+struct LoraMultiBwdScratch {
+  LoraBwdScratch one[ARTK_LORA_MULTI_MAX];  // per projection: Bt, At, gb16, rowp_g, colp_g (gb, colp_x unused)
+  float* gb_cat;   // [T, r_total]: g_i B_i side by side, the Y of the pass over x
+  float* colp_x;   // [n_slabs][in][r_total]
+  float* dummy;
+  StatsGeom gx;
+  int r_total;
+};
+static void carve_lora_multi_bwd(Workspace& ws, int64_t T, int64_t in, const artk_lora_proj_t* proj, int n,
+                                 LoraMultiBwdScratch& c) {
+  c.r_total = 0;
+  for (int i = 0; i < n; ++i) c.r_total += proj[i].r;
+  for (int i = 0; i < n; ++i) {
+    const int64_t out = proj[i].out;
+    const int r = proj[i].r, RP = round16(r);
+    LoraBwdScratch& o = c.one[i];
+    o.gg = stats_geom(T, out, r);
+    o.Bt = ws.take<uint16_t>((size_t)r * out);
+    o.At = ws.take<uint16_t>((size_t)in * r);
+    o.gb16 = ws.take<uint16_t>((size_t)T * RP);
+    o.rowp_g = ws.take<float>((size_t)o.gg.n_chunks * T * r);
+    o.colp_g = ws.take<float>((size_t)o.gg.n_slabs * out * r);
+  }
+  c.gx = stats_geom(T, in, c.r_total);
+  c.gb_cat = ws.take<float>((size_t)T * c.r_total);
+  c.colp_x = ws.take<float>((size_t)c.gx.n_slabs * in * c.r_total);
+  c.dummy = ws.take<float>(1024);
+}
+
+size_t artk_lora_linear_multi_bwd_workspace_bytes(int64_t T, int64_t in, const artk_lora_proj_t* proj,
+                                                  int32_t n) {
+  if (proj == nullptr || n < 1 || n > ARTK_LORA_MULTI_MAX) return 0;
+  Workspace ws(nullptr, 0);
+  LoraMultiBwdScratch c;
+  carve_lora_multi_bwd(ws, T, in, proj, n, c);
+  return ws.used + 256;
+}
+
+int32_t artk_lora_linear_multi_bwd(const void* x, const artk_lora_proj_t* proj, int32_t n, float scale,
+                                   int64_t T, int64_t in, void* dx, void* workspace, size_t workspace_bytes,
+                                   artk_stream_t stream) {
+  int32_t rc = check_multi(proj, n, T, in, true);
+  if (rc) return rc;
+  ARTK_CHECK_ARG(x != nullptr && dx != nullptr && aligned16(x) && aligned16(dx),
+                 "x and dx must be 16-byte aligned pointers");
+  Workspace ws(workspace, workspace_bytes);
+  LoraMultiBwdScratch c;
+  carve_lora_multi_bwd(ws, T, in, proj, n, c);
+  if (!ws.ok()) {
+    set_error("workspace too small: need %zu bytes, got %zu", ws.used, workspace_bytes);
+    return ARTK_ERR_WORKSPACE_TOO_SMALL;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  LoraMultiParams p;
+  p.N = T;
+  p.NT = (int)((T + TILE - 1) / TILE);
+  p.n_jobs = 1;
+  const int MT = (int)((in + TILE - 1) / TILE);
+  p.job[0] = LoraJob{(uint16_t*)dx, nullptr, in, MT, 0, 0, n};
+  p.n_tiles = MT * p.NT;
+  StatsReduceJob jx{c.colp_x, c.gx.n_slabs, in, scale, nullptr, 1, nullptr, 0, 0.f};
+  jx.n_split = n;
+  int r0 = 0;
+  for (int i = 0; i < n; ++i) {
+    const artk_lora_proj_t& q = proj[i];
+    LoraBwdScratch& o = c.one[i];
+    const int RP = round16(q.r);
+    if ((rc = launch_small_transpose2(q.B, o.Bt, 1, q.out, q.r, q.A, o.At, 1, q.r, in, st))) return rc;
+    // one pass over g_i: partials of g_i B_i (over column chunks) and of g_i^T (x A_i^T) (over row slabs)
+    if ((rc = launch_stats(q.g, T, q.out, o.Bt, q.xa, q.r, o.gg, o.rowp_g, o.colp_g, c.dummy, st))) return rc;
+    StatsReduceJob ja{o.rowp_g, o.gg.n_chunks, T, 1.f, c.gb_cat, 0, o.gb16, RP, scale};
+    ja.out_ld = c.r_total;
+    ja.out_off = r0;
+    StatsReduceJob jb{o.colp_g, o.gg.n_slabs, q.out, scale, q.dB, 0, nullptr, 0, 0.f};
+    if ((rc = launch_stats_reduce(ja, jb, q.r, st))) return rc;
+    p.seg[i] = LoraSeg{q.W_t, q.g, o.At, o.gb16, q.out, q.r, RP};
+    jx.outs[i] = q.dA;
+    jx.e_start[i] = r0;
+    r0 += q.r;
+  }
+  jx.e_start[n] = r0;
+  // dx = sum_i ( g_i W_i + (s g_i B_i) A_i ): one launch, the projections as K segments
+  if ((rc = launch_lora_multi(p, st))) return rc;
+  // one pass over x: [dA_0; dA_1; ...] = s [g_0 B_0 | g_1 B_1 | ...]^T x
+  if ((rc = launch_stats(x, T, in, nullptr, c.gb_cat, c.r_total, c.gx, nullptr, c.colp_x, c.dummy, st))) return rc;
+  StatsReduceJob none{nullptr, 0, 0, 0.f, nullptr, 0, nullptr, 0, 0.f};
+  return launch_stats_reduce(jx, none, c.r_total, st);
 }
 
 // ---- the same linear with the frozen weight kept as NF4 codes -------------------------------

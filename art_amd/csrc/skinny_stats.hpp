@@ -334,6 +334,14 @@ struct StatsReduceJob {
   uint16_t* out_bf16;
   int RP;
   float bf16_scale;
+  // plain (not transposed) output: row pitch and first column of the R results inside a wider
+  // [n][out_ld] array (0: dense [n][R])
+  int out_ld = 0, out_off = 0;
+  // transposed output split over several arrays: results e_start[i] <= e < e_start[i+1] go to
+  // outs[i] as [e - e_start[i]][n] (n_split == 0: everything to `out`)
+  int n_split = 0;
+  float* outs[4] = {nullptr, nullptr, nullptr, nullptr};
+  int e_start[5] = {0, 0, 0, 0, 0};
 };
 
 __global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob a, StatsReduceJob b, int R, int nblk_a) {
@@ -357,8 +365,17 @@ __global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob
       for (int u = 0; u < 8; ++u) s += v[u];
     }
     s *= j.scale;
-    if (j.transposed) j.out[(int64_t)e * j.n + row] = s;
-    else j.out[row * R + e] = s;
+    if (j.transposed) {
+      if (j.n_split > 0) {
+        int k = 0;
+        while (k + 1 < j.n_split && e >= j.e_start[k + 1]) ++k;
+        j.outs[k][(int64_t)(e - j.e_start[k]) * j.n + row] = s;
+      } else {
+        j.out[(int64_t)e * j.n + row] = s;
+      }
+    } else {
+      j.out[row * (j.out_ld ? j.out_ld : R) + j.out_off + e] = s;
+    }
   }
   if (j.out_bf16) j.out_bf16[row * j.RP + e] = f32_to_bf16(s * j.bf16_scale);
 }

@@ -134,73 +134,69 @@ class LoRALinear(nn.Module):
 
 
 class _FusedLoRAFn(torch.autograd.Function):
-    """Several projections of the same input as ONE product: the frozen weights
-    are concatenated along the output dimension, the adapters become a rank
-    sum(r_i) update whose B factor is block-diagonal."""
+    """Several projections of the same input through the library's multi-projection entry
+    points: one launch walks the tiles of all of them over one x, the input gradient is one
+    accumulation over all of them.  Weights, adapters, outputs and upstream gradients stay
+    separate tensors: nothing is concatenated and no block-diagonal factor is built."""
 
     @staticmethod
-    def forward(ctx, x, weight_cat, bias_cat, scale, outs, ranks, *AB):
+    def forward(ctx, x, scale, n, *rest):
+        weights, biases = rest[:n], rest[n:2 * n]
+        As, Bs = rest[2 * n:3 * n], rest[3 * n:4 * n]
         lead = x.shape[:-1]
-        n = len(outs)
-        As, Bs = AB[:n], AB[n:]
         x2 = x.reshape(-1, x.shape[-1]).to(torch.bfloat16).contiguous()
-        A_cat = torch.cat([a.detach().to(torch.bfloat16) for a in As], 0).contiguous()
-        B_bd = torch.zeros((sum(outs), sum(ranks)), dtype=torch.bfloat16, device=x.device)
-        o0 = r0 = 0
-        for b, o, r in zip(Bs, outs, ranks):
-            B_bd[o0:o0 + o, r0:r0 + r] = b.detach().to(torch.bfloat16)
-            o0 += o
-            r0 += r
-        y, xa = ops.lora_linear_fwd(x2, weight_cat, A_cat, B_bd, scale, bias_cat)
-        ctx.save_for_backward(x2, weight_cat, A_cat, B_bd, xa)
-        ctx.meta = (scale, lead, outs, ranks, [a.dtype for a in As], [b.dtype for b in Bs], x.dtype)
-        return y.view(*lead, sum(outs))
+        A16 = [a.detach().to(torch.bfloat16).contiguous() for a in As]
+        B16 = [b.detach().to(torch.bfloat16).contiguous() for b in Bs]
+        ys, xas = ops.lora_linear_multi_fwd(x2, list(weights), A16, B16, scale, list(biases))
+        ctx.save_for_backward(x2, *weights, *A16, *B16, *xas)
+        ctx.meta = (scale, n, lead, [a.dtype for a in As], [b.dtype for b in Bs], x.dtype)
+        return tuple(y.view(*lead, y.shape[-1]) for y in ys)
 
     @staticmethod
-    def backward(ctx, g):
-        x2, weight_cat, A_cat, B_bd, xa = ctx.saved_tensors
-        scale, lead, outs, ranks, a_dt, b_dt, x_dt = ctx.meta
-        g2 = g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous()
-        dx, dA, dB = ops.lora_linear_bwd(g2, x2, ops.transposed_weight(weight_cat), A_cat, B_bd, xa, scale)
-        dAs, dBs = [], []
-        o0 = r0 = 0
-        for o, r, ad, bd in zip(outs, ranks, a_dt, b_dt):
-            dAs.append(dA[r0:r0 + r].to(ad))
-            dBs.append(dB[o0:o0 + o, r0:r0 + r].to(bd))   # off-diagonal blocks belong to no adapter
-            o0 += o
-            r0 += r
-        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, None, None, None, *dAs, *dBs)
+    def backward(ctx, *gs):
+        scale, n, lead, a_dt, b_dt, x_dt = ctx.meta
+        saved = ctx.saved_tensors
+        x2 = saved[0]
+        weights, A16, B16, xas = (saved[1 + k * n:1 + (k + 1) * n] for k in range(4))
+        g2 = []
+        for g, w in zip(gs, weights):   # an output nobody used has no gradient: zeros
+            g2.append(torch.zeros((x2.shape[0], w.shape[0]), dtype=torch.bfloat16, device=x2.device) if g is None
+                      else g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous())
+        dx, dAs, dBs = ops.lora_linear_multi_bwd(g2, x2, [ops.transposed_weight(w) for w in weights], list(A16),
+                                                 list(B16), list(xas), scale)
+        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, *([None] * (2 * n)),
+                *[d.to(t) for d, t in zip(dAs, a_dt)], *[d.to(t) for d, t in zip(dBs, b_dt)])
 
 
 class FusedLoRALinear(nn.Module):
-    """Projections that read the same activations (q/k/v, or gate/up) as one
-    product: one pass over x instead of one per projection, and the narrow
-    projections (k, v: 256 or 512 columns) ride in the tiles of the wide one
-    instead of leaving most of the GPU idle.  ``forward(x)`` returns the tuple of
-    the individual outputs; the parameters stay per projection."""
+    """Projections that read the same activations (q/k/v, or gate/up) in one call each way:
+    one persistent launch over the tiles of all of them (the narrow projections, k and v with
+    256 or 512 columns, ride along with the wide one instead of leaving most of the GPU idle),
+    one accumulation for the input gradient, one pass over x for all dA.  ``forward(x)``
+    returns the tuple of the individual outputs.  The module holds the given layers and
+    nothing else: no second copy of the frozen weights, no stacked adapters."""
 
     def __init__(self, layers):
         super().__init__()
         layers = list(layers)
         if len({l.in_features for l in layers}) != 1 or len({l.scaling for l in layers}) != 1:
             raise ValueError("fused projections need the same input size and scaling")
+        if not 1 <= len(layers) <= 4:
+            raise ValueError("one to four projections per call")
+        if any(l.weight is None for l in layers):
+            raise ValueError("fused projections need bf16 base weights (not NF4 codes)")
         self.outs = tuple(l.out_features for l in layers)
         self.ranks = tuple(l.r for l in layers)
         if sum(self.ranks) > 64:
             raise ValueError("sum of ranks above 64")
         self.scaling = layers[0].scaling
-        self.weight = nn.Parameter(torch.cat([l.weight.detach() for l in layers], 0).contiguous(),
-                                   requires_grad=False)
-        if any(l.bias is not None for l in layers):   # frozen biases; projections without one add zero
-            parts = [l.bias.detach() if l.bias is not None else
-                     torch.zeros(l.out_features, dtype=torch.bfloat16, device=l.weight.device) for l in layers]
-            self.bias = nn.Parameter(torch.cat(parts).to(torch.bfloat16).contiguous(), requires_grad=False)
-        else:
-            self.bias = None
-        self.lora_A = nn.ParameterList([l.lora_A for l in layers])
-        self.lora_B = nn.ParameterList([l.lora_B for l in layers])
+        self.layers = nn.ModuleList(layers)
 
     def forward(self, x: torch.Tensor):
-        y = _FusedLoRAFn.apply(x, self.weight, self.bias, float(self.scaling), self.outs, self.ranks,
-                               *self.lora_A, *self.lora_B)
-        return torch.split(y, self.outs, dim=-1)
+        ls = self.layers
+        for l in ls:
+            if l.bias is not None and l.bias.requires_grad:
+                raise ValueError("the bias of a LoRA-wrapped linear is frozen (peft bias='none')")
+        biases = [None if l.bias is None else l.bias.detach().to(torch.bfloat16).contiguous() for l in ls]
+        return _FusedLoRAFn.apply(x, float(self.scaling), len(ls), *[l.weight for l in ls], *biases,
+                                  *[l.lora_A for l in ls], *[l.lora_B for l in ls])

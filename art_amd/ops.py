@@ -220,7 +220,9 @@ def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask
     """One call for loss and d_hidden of a packed batch given its hidden states.
 
     All per-token inputs are the un-shifted PackedTensors rows flattened to [T].
-    Returns (scalars f32 [4], logprob f32 [T], d_hidden bf16 [T,H]).  With
+    Returns (scalars f32 [5] = (loss, mean_policy_loss, mean_kl, mask_count, dropped_rows),
+    logprob f32 [T], d_hidden bf16 [T,H]).  dropped_rows counts rows whose target has
+    probability below e^-80 under the current policy: their d_hidden row is zero.  With
     skip_inactive the lm_head projection runs only for positions that can
     contribute to the loss; logprob is NaN elsewhere."""
     T, H = hidden.shape
@@ -238,11 +240,12 @@ def grpo_fused(hidden, lm_head, lm_head_t, tokens, old_logprob, advantages, mask
     lib = _lib.load()
     dev = hidden.device
     if out is None:
-        scalars = torch.empty(4, dtype=torch.float32, device=dev)
+        scalars = torch.empty(5, dtype=torch.float32, device=dev)
         logprob = torch.empty(T, dtype=torch.float32, device=dev)
         d_hidden = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     else:
         scalars, logprob, d_hidden = out
+        _need(scalars, "scalars", torch.float32, (5,))
     need = lib.artk_grpo_fused_workspace_bytes(T, V, H, chunk_tokens)
     ws = workspace if workspace is not None else _workspace(need, dev)
     _lib.check(
@@ -533,6 +536,76 @@ def _nf4_struct(w) -> "_lib.Nf4Struct":
                           float(w.offset), int(w.blocksize))
 
 
+def _lora_proj_array(projs):
+    """ctypes array of artk_lora_proj_t from dicts of tensors (missing keys: NULL)."""
+    arr = (_lib.LoraProjStruct * len(projs))()
+    for st, d in zip(arr, projs):
+        for key in ("W", "W_t", "A", "B", "bias", "y", "g", "xa", "dA", "dB"):
+            t = d.get(key)
+            setattr(st, key, None if t is None else t.data_ptr())
+        st.out, st.r = d["B"].shape
+    return arr
+
+
+def lora_linear_multi_fwd(x, Ws, As, Bs, scale: float, biases=None):
+    """Projections of the same x in one call: for each i, (y_i bf16 [T,out_i], xa_i f32 [T,r_i]) with
+    y_i = x W_i^T + bias_i + scale (x A_i^T) B_i^T.  Nothing is concatenated: every projection keeps
+    its own weight, factors and output.  Returns (ys, xas)."""
+    T, n_in = x.shape
+    n = len(Ws)
+    biases = biases if biases is not None else [None] * n
+    _need(x, "x", torch.bfloat16)
+    dev = x.device
+    projs, ys, xas = [], [], []
+    for W, A, B, bias in zip(Ws, As, Bs, biases):
+        n_out, r = B.shape
+        _need(W, "W", torch.bfloat16, (n_out, n_in))
+        _need(A, "A", torch.bfloat16, (r, n_in))
+        _need(B, "B", torch.bfloat16, (n_out, r))
+        if bias is not None:
+            _need(bias, "bias", torch.bfloat16, (n_out,))
+        y = torch.empty((T, n_out), dtype=torch.bfloat16, device=dev)
+        xa = torch.empty((T, r), dtype=torch.float32, device=dev)
+        ys.append(y)
+        xas.append(xa)
+        projs.append({"W": W, "A": A, "B": B, "bias": bias, "y": y, "xa": xa})
+    arr = _lora_proj_array(projs)
+    lib = _lib.load()
+    ws = _workspace(lib.artk_lora_linear_multi_fwd_workspace_bytes(T, n_in, arr, n), dev)
+    _lib.check(lib.artk_lora_linear_multi_fwd(x.data_ptr(), arr, n, scale, T, n_in, ws.data_ptr(), ws.numel(),
+                                              _stream(dev)))
+    return ys, xas
+
+
+def lora_linear_multi_bwd(gs, x, W_ts, As, Bs, xas, scale: float):
+    """Backward of lora_linear_multi_fwd: (dx bf16 [T,in], [dA_i f32 [r_i,in]], [dB_i f32 [out_i,r_i]]) for
+    the upstream gradients g_i bf16 [T,out_i]; dx is the sum over the projections."""
+    T, n_in = x.shape
+    n = len(gs)
+    _need(x, "x", torch.bfloat16)
+    dev = x.device
+    projs, dAs, dBs = [], [], []
+    for g, W_t, A, B, xa in zip(gs, W_ts, As, Bs, xas):
+        n_out, r = B.shape
+        _need(g, "g", torch.bfloat16, (T, n_out))
+        _need(W_t, "W_t", torch.bfloat16, (n_in, n_out))
+        _need(A, "A", torch.bfloat16, (r, n_in))
+        _need(B, "B", torch.bfloat16, (n_out, r))
+        _need(xa, "xa", torch.float32, (T, r))
+        dA = torch.empty((r, n_in), dtype=torch.float32, device=dev)
+        dB = torch.empty((n_out, r), dtype=torch.float32, device=dev)
+        dAs.append(dA)
+        dBs.append(dB)
+        projs.append({"W_t": W_t, "A": A, "B": B, "g": g, "xa": xa, "dA": dA, "dB": dB})
+    arr = _lora_proj_array(projs)
+    lib = _lib.load()
+    dx = torch.empty((T, n_in), dtype=torch.bfloat16, device=dev)
+    ws = _workspace(lib.artk_lora_linear_multi_bwd_workspace_bytes(T, n_in, arr, n), dev)
+    _lib.check(lib.artk_lora_linear_multi_bwd(x.data_ptr(), arr, n, scale, T, n_in, dx.data_ptr(), ws.data_ptr(),
+                                              ws.numel(), _stream(dev)))
+    return dx, dAs, dBs
+
+
 def lora_linear_fwd_nf4(x, w_nf4, A, B, scale: float, bias: Optional[torch.Tensor] = None):
     """lora_linear_fwd with the frozen weight given as NF4 codes (art_amd.quant.NF4Weight); the
     bf16 weight lives in the call's workspace only."""
@@ -683,3 +756,23 @@ def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> int:
         raise ValueError("src and dst differ in size")
     _lib.check(_lib.load().artk_stream_copy(src.data_ptr(), dst.data_ptr(), nbytes, _stream(src.device)))
     return nbytes
+
+
+def lds_probe(waves: int, kind: int, reads_per_dma: int, iters: int, blocks: int,
+              device: torch.device) -> dict:
+    """Runs the LDS bandwidth probe and synchronises.  ``kind``: 0 ds_read_b128 contiguous, 1 ds_read_b128
+    in the GEMM's fragment pattern, 2 ds_read_b64_tr_b16.  Returns the read (and DMA-written) bytes per
+    core clock and CU (median over the work-groups) and the core clock in GHz seen by the probe."""
+    src = torch.zeros(65536, dtype=torch.uint8, device=device)
+    cyc = torch.zeros(blocks, 2, dtype=torch.int64, device=device)
+    _lib.check(_lib.load().artk_lds_probe(int(waves), int(kind), int(reads_per_dma), src.data_ptr(), int(iters),
+                                          int(blocks), cyc.data_ptr(), _stream(device)))
+    torch.cuda.synchronize(device)
+    c = cyc.cpu()
+    core = float(c[:, 0].median())
+    ticks = float(c[:, 1].median())
+    read_bytes = float(waves) * iters * 16 * (512 if kind == 2 else 1024)
+    n_dma = 0 if reads_per_dma == 0 else len([j for j in range(16) if j % reads_per_dma == reads_per_dma - 1])
+    write_bytes = float(waves) * iters * n_dma * 1024
+    return {"read_B_per_clk": read_bytes / core, "dma_write_B_per_clk": write_bytes / core,
+            "core_GHz": core / (ticks * 10.0) if ticks > 0 else None}

@@ -201,15 +201,37 @@ def fused_grpo_loss(hidden_states, lm_head, tokens, logprobs, advantages, assist
     ``skip_inactive``: project only the positions whose loss term can be
     non-zero (the reference projects all of them and multiplies by the mask,
     train.py:145-151); loss, metrics and gradient are unchanged, new_logprobs is
-    NaN at the skipped positions."""
+    NaN at the skipped positions.
+
+    metrics["dropped_rows"] counts positions whose sampled token has probability below
+    e^-80 under the current policy: their gradient row is zero (see artk_grpo_fused).
+
+    When no gradient can be asked for (``torch.no_grad()`` / ``inference_mode``, or hidden
+    states that do not require grad) only the forward half runs: the lm_head projection
+    without the stash of exponentials, then the loss kernels; no d_hidden GEMM.  Loss and
+    logprobs are the same numbers; ``skip_inactive`` has no effect there."""
     clip_lo, clip_hi = ops.clip_bounds(epsilon, epsilon_high)
     ref = ref_logprobs if beta > 0.0 else None
     hidden = hidden_states.to(torch.bfloat16).contiguous()
+    if not (torch.is_grad_enabled() and hidden_states.requires_grad):
+        B, S, H = hidden.shape
+        T = B * S
+        flat = lambda t: None if t is None else t.reshape(T).contiguous()
+        logprob, _ = ops.logprob_fwd(hidden.reshape(T, H), lm_head, flat(tokens), True, S)
+        scalars, _ = ops.grpo_loss(
+            logprob, flat(logprobs.to(torch.float32)), flat(advantages.to(torch.float32)),
+            flat(assistant_mask), flat(weights.to(torch.float32)),
+            None if ref is None else flat(ref.to(torch.float32)), True, S, clip_lo, clip_hi,
+            float(beta), want_coef=False)
+        metrics = {"policy_loss": scalars[1], "kl_div": scalars[2], "mask_count": scalars[3],
+                   "dropped_rows": torch.zeros((), dtype=torch.float32, device=hidden.device)}
+        return scalars[0], metrics, logprob.view(B, S)
     loss, scalars, logprob = _FusedGRPOLossFn.apply(
         hidden, lm_head, tokens, logprobs.to(torch.float32), advantages.to(torch.float32),
         assistant_mask, weights.to(torch.float32), None if ref is None else ref.to(torch.float32),
         clip_lo, clip_hi, float(beta), chunk_tokens, bool(skip_inactive))
-    return loss, {"policy_loss": scalars[1], "kl_div": scalars[2], "mask_count": scalars[3]}, logprob
+    return loss, {"policy_loss": scalars[1], "kl_div": scalars[2], "mask_count": scalars[3],
+                  "dropped_rows": scalars[4]}, logprob
 
 
 def calculate_attn_bias(batch_size, seq_len, device, group_ids, parent_ids, autocast_dtype):
@@ -290,6 +312,9 @@ def get_compute_loss_fn(trainer) -> Callable[..., torch.Tensor]:
         trainer._metrics["policy_loss"].append(metrics["policy_loss"].detach())
         if config.beta > 0.0:
             trainer._metrics["kl_div"].append(metrics["kl_div"].detach())
+        # no counterpart in the reference: positions whose gradient row was dropped because the
+        # sampled token has probability below e^-80 under the current policy (0 in a healthy run)
+        trainer._metrics["dropped_rows"].append(metrics["dropped_rows"].detach())
         return loss
 
     return compute_loss

@@ -32,6 +32,10 @@ TRAFFIC_BYTES = {"c3": 2.05e10, "c1": None}
 # moe_gemm_kernel, mean bytes per launch over the 4 launches of the step with gate|up fused (FETCH_SIZE x 2 KiB +
 # WRITE_SIZE x 1 KiB, the factors a 1 GiB copy gives): 949 MB read + 210 MB written
 MOE_TRAFFIC_BYTES = 1.16e9
+# lora_multi_gemm_kernel on the gate|up forward (8192 x 2048 -> 11008 + 11008): filled in from
+# profiles/lora_c2_pmc.md
+LORA_TRAFFIC_BYTES = None
+LORA_TRAFFIC_SOURCE = None
 MOE_TRAFFIC_SOURCE = ("profiles/moe_c5_kernel_trace.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of "
                       "this command, scaled by a 1 GiB copy; not measured in this run)")
 TRAFFIC_SOURCE = {"c3": "profiles/lmhead_fwd_c3_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier "
@@ -170,23 +174,29 @@ def base_result(args, metric, unit, value, ms_per_step, workload):
 def bench_lora(args):
     """LoRA linear fwd+bwd over the six projections of one Qwen2.5-3B layer that have
     in = 2048 (q, o: out 2048; k, v: out 256; gate, up: out 11008), T = 8192, r = 8, alpha = 16.
-    One step = forward + backward of all six.  `value` = algorithmic TFLOP/s of the step when the
-    projections that read the same activations run as one product (q/k/v and gate/up, the way
-    art_amd.lora.FusedLoRALinear runs them: weights concatenated along the output dimension,
-    adapters stacked with a block-diagonal B); `separate` = the same six as six calls."""
+    One step = forward + backward of all six.  `value` = algorithmic TFLOP/s of the step as a user
+    runs it: the modules of art_amd.lora (FusedLoRALinear for q|k|v and for gate|up, LoRALinear for o)
+    called through torch autograd with one upstream gradient tensor per projection; the projections
+    that read the same activations go through the library's multi-projection entry points (separate
+    weights, adapters, outputs and gradients; nothing concatenated).  `raw_multi` = the same entry
+    points called directly; `raw_concatenated` = the single-projection entry points on
+    pre-concatenated weights / stacked adapters / concatenated upstream gradients (built outside the
+    timed region); `separate` = six single-projection calls."""
     import math
 
     import torch
 
     from art_amd import ops
+    from art_amd.lora import FusedLoRALinear, LoRALinear
 
     dev = torch.device("cuda:0")
     T, n_in, r, scale = 8192, 2048, 8, 2.0
     g = torch.Generator().manual_seed(1002)
     x_cpu = torch.randn(T, n_in, generator=g).to(torch.bfloat16)
     x = x_cpu.to(dev)
+    names = ("q", "o", "k", "v", "gate", "up")
     cpu, shapes = {}, {}
-    for name, n_out in (("q", 2048), ("o", 2048), ("k", 256), ("v", 256), ("gate", 11008), ("up", 11008)):
+    for name, n_out in zip(names, (2048, 2048, 256, 256, 11008, 11008)):
         W = (0.02 * torch.randn(n_out, n_in, generator=g)).to(torch.bfloat16)
         A = ((torch.rand(r, n_in, generator=g) * 2 - 1) / math.sqrt(n_in)).to(torch.bfloat16)
         B = (0.01 * torch.randn(n_out, r, generator=g)).to(torch.bfloat16)
@@ -202,8 +212,16 @@ def bench_lora(args):
         y, xa = ops.lora_linear_fwd(x, W, A, B, scale)
         return (y,) + ops.lora_linear_bwd(up, x, Wt, A, B, xa, scale)
 
-    def fuse(names):
-        parts = [shapes[n] for n in names]
+    def multi(group):
+        parts = [shapes[n] for n in group]
+        ys, xas = ops.lora_linear_multi_fwd(x, [p[1] for p in parts], [p[3] for p in parts],
+                                            [p[4] for p in parts], scale)
+        dx, dAs, dBs = ops.lora_linear_multi_bwd([p[5] for p in parts], x, [p[2] for p in parts],
+                                                 [p[3] for p in parts], [p[4] for p in parts], xas, scale)
+        return ys, dx, dAs, dBs
+
+    def fuse(group):
+        parts = [shapes[n] for n in group]
         W = torch.cat([p[1] for p in parts], 0).contiguous()
         A = torch.cat([p[3] for p in parts], 0).contiguous()
         B = torch.zeros(W.shape[0], A.shape[0], dtype=torch.bfloat16, device=dev)
@@ -214,53 +232,92 @@ def bench_lora(args):
         up = torch.cat([p[5] for p in parts], 1).contiguous()
         return (W.shape[0], W, ops.transpose(W), A, B, up)
 
-    fused = {"qkv": fuse(("q", "k", "v")), "o": shapes["o"], "gate_up": fuse(("gate", "up"))}
+    # the modules a user holds: one LoRALinear per projection (adapters in bf16, as peft keeps them
+    # under the reference's bf16 training), grouped by the activations they read
+    mods = {}
+    for name in names:
+        n_out, Wd, _, Ad, Bd, _ = shapes[name]
+        m = LoRALinear(n_in, n_out, r=r, lora_alpha=int(scale * r), device=dev, dtype=torch.bfloat16)
+        with torch.no_grad():
+            m.weight.copy_(Wd)
+            m.lora_A.copy_(Ad)
+            m.lora_B.copy_(Bd)
+        mods[name] = m
+    groups = (("q", "k", "v"), ("o",), ("gate", "up"))
+    fused_mods = [FusedLoRALinear([mods[n] for n in grp]) for grp in groups]
+    ups = [[shapes[n][5] for n in grp] for grp in groups]
+    xg = x.detach().requires_grad_(True)
+    params = [p for m in mods.values() for p in (m.lora_A, m.lora_B)]
+    for m in fused_mods:   # transposed copies of the frozen weights are made once per weight version
+        for l in m.layers:
+            ops.transposed_weight(l.weight)
+
+    def step_module():
+        xg.grad = None
+        for p_ in params:
+            p_.grad = None
+        for m, u in zip(fused_mods, ups):
+            torch.autograd.backward(m(xg), u)
+
+    def step_raw_multi():
+        for grp in groups:
+            multi(grp)
 
     def step_separate():
         for sh in shapes.values():
             one(sh)
 
-    def step_fused():
-        for sh in fused.values():
-            one(sh)
-
+    dt = timed(step_module, args.steps, args.warmup)
+    dt_raw = timed(step_raw_multi, args.steps, args.warmup)
+    per_group = {}
+    for grp in (("q", "k", "v"), ("gate", "up")):
+        fl = sum(flops(shapes[m][0]) for m in grp)
+        gdt = timed(lambda: multi(grp), args.steps, args.warmup)
+        per_group["|".join(grp)] = {"us_fwd_bwd": gdt * 1e6, "tflops": fl / gdt / 1e12,
+                                    "frac": fl / gdt / 1e12 / PEAK_BF16_TFLOPS}
     per_shape = {}
     for name in ("q", "k", "gate"):
         sh = shapes[name]
-        dt = timed(lambda: one(sh), args.steps, args.warmup)
-        per_shape[f"out={sh[0]}"] = {"us_fwd_bwd": dt * 1e6, "tflops": flops(sh[0]) / dt / 1e12,
-                                     "frac": flops(sh[0]) / dt / 1e12 / PEAK_BF16_TFLOPS}
-    per_fused = {}
-    for name, members in (("qkv", ("q", "k", "v")), ("gate_up", ("gate", "up"))):
-        sh = fused[name]
-        fl = sum(flops(shapes[m][0]) for m in members)
-        dt = timed(lambda: one(sh), args.steps, args.warmup)
-        per_fused[name] = {"out": sh[0], "rank": len(members) * r, "us_fwd_bwd": dt * 1e6,
-                           "tflops": fl / dt / 1e12, "frac": fl / dt / 1e12 / PEAK_BF16_TFLOPS}
+        sdt = timed(lambda: one(sh), args.steps, args.warmup)
+        per_shape[f"out={sh[0]}"] = {"us_fwd_bwd": sdt * 1e6, "tflops": flops(sh[0]) / sdt / 1e12,
+                                     "frac": flops(sh[0]) / sdt / 1e12 / PEAK_BF16_TFLOPS}
     dt_sep = timed(step_separate, args.steps, args.warmup)
-    dt = timed(step_fused, args.steps, args.warmup)
+    cat = {"qkv": fuse(("q", "k", "v")), "o": shapes["o"], "gate_up": fuse(("gate", "up"))}
+    dt_cat = timed(lambda: [one(sh) for sh in cat.values()], args.steps, args.warmup)
+    cat_bytes = sum(sh[1].numel() * 2 * 2 + sh[5].numel() * 2 for k_, sh in cat.items() if k_ != "o")
+    del cat
     # dominant kernel, from a separate burst with the library's HIP-event brackets on
     ops.profile_enable(True)
     for _ in range(args.steps):
-        one(fused["gate_up"])
+        multi(("gate", "up"))
     torch.cuda.synchronize()
     gemm_ms, gemm_n = ops.profile_collect(ops.PROF_LORA_GEMM)
     ops.profile_enable(False)
     res = base_result(args, "LoRA linear fwd+bwd TFLOP/s (Qwen2.5-3B shapes)", "TFLOP/s", total / dt / 1e12,
                       dt * 1e3, "C2-lora-qwen2.5-3b")
     res["config"].update({"tokens": T, "in": n_in, "rank": r, "projections": "q,o,k,v,gate,up",
-                          "path": "q/k/v and gate/up as one product each (FusedLoRALinear), o alone"})
+                          "path": "art_amd.lora modules under torch autograd: FusedLoRALinear(q,k,v), "
+                                  "LoRALinear(o), FusedLoRALinear(gate,up); one upstream gradient per projection"})
     res["frac_of_bf16_peak"] = total / dt / 1e12 / PEAK_BF16_TFLOPS
-    res["fused_products"] = per_fused
+    res["raw_multi"] = {"value": total / dt_raw / 1e12, "unit": "TFLOP/s", "ms_per_step": dt_raw * 1e3,
+                        "frac_of_bf16_peak": total / dt_raw / 1e12 / PEAK_BF16_TFLOPS, "groups": per_group,
+                        "note": "artk_lora_linear_multi_fwd/_bwd called directly: q|k|v, o, gate|up"}
+    res["raw_concatenated"] = {"value": total / dt_cat / 1e12, "unit": "TFLOP/s", "ms_per_step": dt_cat * 1e3,
+                               "extra_resident_bytes": cat_bytes,
+                               "note": "single-projection entry points on weights, transposed weights and upstream "
+                                       "gradients concatenated outside the timed region (extra_resident_bytes of "
+                                       "copies), adapters stacked with a block-diagonal B"}
     res["separate"] = {"value": total / dt_sep / 1e12, "unit": "TFLOP/s", "ms_per_step": dt_sep * 1e3,
                        "frac_of_bf16_peak": total / dt_sep / 1e12 / PEAK_BF16_TFLOPS, "shapes": per_shape,
                        "note": "six separate calls; per shape: one projection fwd+bwd"}
     launch_ms = gemm_ms / max(gemm_n, 1)
     ach = 2.0 * T * n_in * 22016 / (launch_ms * 1e-3) / 1e12
-    res["roofline"] = {"kernel": "lora_gemm_kernel (fused gate/up: mean of the y and dx launches)",
+    res["roofline"] = {"kernel": "lora_multi_gemm_kernel (gate|up: mean of the y launch and the dx launch)",
                        "bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "launch_ms": launch_ms,
-                       "flop_per_launch": 2.0 * T * n_in * 22016}
+                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": LORA_TRAFFIC_BYTES,
+                       "traffic_source": LORA_TRAFFIC_SOURCE, "launch_ms": launch_ms,
+                       "flop_per_launch": 2.0 * T * n_in * 22016,
+                       "algorithmic_bytes": 2.0 * (T * n_in + T * 22016 + n_in * 22016)}
     if not args.no_secondary:
         # The LoRA linear the way peft evaluates it, in stock torch ops on the same GPU:
         # base(x) + scale * lora_B(lora_A(x)), autograd for dx, dA, dB (W frozen).
@@ -268,9 +325,9 @@ def bench_lora(args):
 
         def torch_step():
             for _, W, _, A, B, up in shapes.values():
-                xg = x.detach().requires_grad_(True)
+                xg_ = x.detach().requires_grad_(True)
                 Ag, Bg = A.detach().requires_grad_(True), B.detach().requires_grad_(True)
-                y = F.linear(xg, W) + scale * F.linear(F.linear(xg, Ag), Bg)
+                y = F.linear(xg_, W) + scale * F.linear(F.linear(xg_, Ag), Bg)
                 y.backward(up)
 
         tdt = timed(torch_step, max(args.steps // 2, 3), 2)
@@ -281,44 +338,51 @@ def bench_lora(args):
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import lora_oracle
 
-        # CPU oracle (fp32) of q, k and v: the timing sample, and the parity reference of this run for
-        # the separate calls (y, dx, dA, dB of q and k) and for the fused q/k/v product (dx is the sum)
+        # CPU oracle (fp32) of all six projections: the timing sample (1 warm-up + 3 runs, median) and the
+        # parity reference of this run for the module step and for the raw multi-projection calls
         ref, times = {}, []
-        for rep in range(4):           # 1 warm-up + 3 runs
+        for rep in range(4):
             t0 = time.perf_counter()
-            for name in ("q", "k", "v"):
+            for name in names:
                 W, A, B, up = cpu[name]
-                ref[name] = lora_oracle.lora_linear_grads(x_cpu, W, A, B, scale, up)
+                out = lora_oracle.lora_linear_grads(x_cpu, W, A, B, scale, up)
+                if rep == 0:
+                    ref[name] = out
             if rep:
                 times.append(time.perf_counter() - t0)
         cdt = sorted(times)[1]
         t0 = time.perf_counter()
-        for name in ("q", "k", "v"):
+        for name in names:
             W, A, B, up = cpu[name]
             lora_oracle.lora_linear_grads(x_cpu, W, A, B, scale, up, dtype=torch.bfloat16)
         cdt16 = time.perf_counter() - t0
-        fl = sum(flops(shapes[n][0]) for n in ("q", "k", "v"))
-        res["cpu_baseline"] = {"value": fl / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        res["cpu_baseline"] = {"value": total / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
                                "kind": "port",
-                               "sample": f"q, k and v projections fwd+bwd, fp32 torch-CPU oracle, 1 warm-up + 3 runs, "
+                               "sample": f"all six projections fwd+bwd, fp32 torch-CPU oracle, 1 warm-up + 3 runs, "
                                          f"median {cdt:.2f} s",
-                               "bf16": {"value": fl / cdt16 / 1e12, "unit": "TFLOP/s",
+                               "bf16": {"value": total / cdt16 / 1e12, "unit": "TFLOP/s",
                                         "sample": f"same in bf16, one run of {cdt16:.2f} s"}}
         rel = lambda a, b: ((a.double().cpu() - b.double()).norm() / b.double().norm()).item()
         parity = {}
         for name in ("q", "k"):
             got = one(shapes[name])
             parity[name] = dict(zip(("y", "dx", "dA", "dB"), (rel(a, b) for a, b in zip(got, ref[name]))))
-        y, dx, dA, dB = one(fused["qkv"])
-        o0 = r0 = 0
-        fq = {"dx": rel(dx, ref["q"][1] + ref["k"][1] + ref["v"][1])}
-        for name in ("q", "k", "v"):
-            n_out = shapes[name][0]
-            fq[f"y_{name}"] = rel(y[:, o0:o0 + n_out], ref[name][0])
-            fq[f"dA_{name}"] = rel(dA[r0:r0 + r], ref[name][2])
-            fq[f"dB_{name}"] = rel(dB[o0:o0 + n_out, r0:r0 + r], ref[name][3])
-            o0, r0 = o0 + n_out, r0 + r
-        parity["fused_qkv"] = fq
+        for grp in (("q", "k", "v"), ("gate", "up")):
+            ys, dx, dAs, dBs = multi(grp)
+            rec = {"dx": rel(dx, sum(ref[n][1] for n in grp))}
+            for i, name in enumerate(grp):
+                rec[f"y_{name}"] = rel(ys[i], ref[name][0])
+                rec[f"dA_{name}"] = rel(dAs[i], ref[name][2])
+                rec[f"dB_{name}"] = rel(dBs[i], ref[name][3])
+            parity["multi_" + "_".join(grp)] = rec
+            del ys, dx, dAs, dBs
+        # the module step itself: x.grad is the sum over all six projections
+        step_module()
+        rec = {"x_grad": rel(xg.grad, sum(ref[n][1] for n in names))}
+        for name in names:
+            rec[f"dA_{name}"] = rel(mods[name].lora_A.grad, ref[name][2])
+            rec[f"dB_{name}"] = rel(mods[name].lora_B.grad, ref[name][3])
+        parity["module_step"] = rec
         parity["tolerance_rel_l2"] = 1e-2
         res["parity_same_run"] = parity
     return res

@@ -66,7 +66,9 @@ int32_t artk_logprob_fwd(const void* hidden, const void* lm_head, const int64_t*
  *   grad_logprob f32 [T]    upstream gradient per position
  *   d_hidden   bf16 [T,H] out
  * Logits are recomputed per chunk of `chunk_tokens` positions into a bounded
- * bf16 scratch inside the workspace.  Requires H % 64 == 0, V % 64 == 0.
+ * bf16 scratch inside the workspace.  A row with a non-zero grad_logprob whose
+ * target has probability below e^-80 gets a zero d_hidden row (see
+ * artk_grpo_fused, which also counts such rows).  Requires H % 64 == 0, V % 64 == 0.
  * ------------------------------------------------------------------------- */
 size_t artk_logprob_bwd_workspace_bytes(int64_t T, int64_t V, int64_t H, int64_t chunk_tokens);
 int32_t artk_logprob_bwd(const void* hidden, const void* lm_head, const void* lm_head_t,
@@ -123,14 +125,17 @@ int32_t artk_grpo_loss_static(const float* new_logprob, const float* old_logprob
  * and target gather (for the rows the backward will read, exp(logit - the
  * target's logit) goes to a bounded bf16 scratch), loss coefficients, d_hidden
  * GEMM of those exponentials against lm_head_t, softmax scaling and one-hot
- * term in its reduction.  A row whose target logit lies more than 88 nats under
- * the row's largest logit (a sampled token of probability < e^-88) overflows the
- * scratch: its d_hidden row is inf / NaN.
+ * term in its reduction.  A row whose target has probability below e^-80 under
+ * the current policy (log-sum-exp more than 80 nats above the target's logit)
+ * would overflow the scratch: its d_hidden row is written as zeros and it is
+ * counted in scalars[4]; its logprob and its loss term are exact.  Every other
+ * row's exponentials are finite by construction, so d_hidden is always finite.
  *   tokens int64 [T], old_logprob/advantages/weights f32 [T], mask u8 [T]:
  *     the un-shifted PackedTensors rows (src/art/local/pack.py:13-21);
  *     the shift of train.py:79,112-117 is applied by index arithmetic.
  *   ref_logprob f32 [T] or NULL   (position frame)
- *   scalars f32 [4] out, logprob f32 [T] out, d_hidden bf16 [T,H] out
+ *   scalars f32 [5] out: {loss, mean_policy_loss, mean_kl, mask_count, dropped_rows}
+ *   logprob f32 [T] out, d_hidden bf16 [T,H] out
  *   flags: 0, or ARTK_FUSED_SKIP_INACTIVE: evaluate the lm_head projection only
  *     for positions that can contribute to the loss (shifted assistant mask set,
  *     weight != 0, and advantage != 0 or a KL term).  The reference computes
@@ -167,6 +172,7 @@ int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t
  *   x bf16 [T,in], W bf16 [out,in] (frozen), A bf16 [r,in], B bf16 [out,r]
  *   bias bf16 [out] or NULL: the frozen bias of the wrapped linear (Qwen2.5 has one on
  *        q/k/v; peft keeps the base layer's bias), added in the GEMM epilogue: y += bias
+ *        (16-byte aligned like every other pointer: it is read with vector loads)
  *   y bf16 [T,out] out, xa f32 [T,r] out (x A^T, kept for the backward)
  * Requires in % 64 == 0, out % 64 == 0, r % 8 == 0, r <= 64.
  * ------------------------------------------------------------------------- */
@@ -379,6 +385,49 @@ int32_t artk_lora_linear_bwd_nf4(const void* g, const void* x, const artk_nf4_t*
                                  size_t workspace_bytes, artk_stream_t stream);
 
 /* ------------------------------------------------------------------------- *
+ * A8, several projections of the same input in one call: q|k|v or gate|up of a
+ * layer.  Replaces: the separate peft lora.Linear modules the reference installs
+ *   on q_proj, k_proj, v_proj (and gate_proj, up_proj), which all read the same
+ *   hidden states (target modules: src/art/dev/model.py:54-62, installed at
+ *   src/art/local/state.py:86-92).  Each projection keeps its own weight, adapter,
+ *   output and gradient arrays: nothing is concatenated, no block-diagonal B is built.
+ * Forward: x A_i^T of all projections in one launch, then ONE persistent GEMM launch
+ *   over the tiles of all projections (narrow k / v ride along with q instead of
+ *   leaving most of the GPU idle).  Writes y_i and xa_i of every projection.
+ * Backward: per projection one pass over g_i (g_i B_i and dB_i); ONE GEMM launch for
+ *   dx = sum_i (g_i W_i + scale (g_i B_i) A_i), the projections being K segments of
+ *   one accumulation, so dx is written once; ONE pass over x for all dA_i.
+ *   Writes dx, dA_i, dB_i; the ranks may add up to 64 at most.
+ * Fields a direction does not use may be NULL.  Same shape rules as the single
+ * projection: in % 64 == 0, out_i % 64 == 0, r_i % 8 == 0; all pointers 16-byte aligned.
+ * ------------------------------------------------------------------------- */
+#define ARTK_LORA_MULTI_MAX 4
+typedef struct artk_lora_proj {
+  const void* W;    /* bf16 [out,in]  frozen weight                (forward)  */
+  const void* W_t;  /* bf16 [in,out]  its transposed copy          (backward) */
+  const void* A;    /* bf16 [r,in]                                 (both)     */
+  const void* B;    /* bf16 [out,r]                                (both)     */
+  const void* bias; /* bf16 [out] or NULL, frozen                  (forward)  */
+  void* y;          /* bf16 [T,out]   out                          (forward)  */
+  const void* g;    /* bf16 [T,out]   upstream gradient of y       (backward) */
+  float* xa;        /* f32 [T,r]      x A^T: out of the forward, in of the backward */
+  float* dA;        /* f32 [r,in]     out                          (backward) */
+  float* dB;        /* f32 [out,r]    out                          (backward) */
+  int64_t out;
+  int32_t r;
+} artk_lora_proj_t;
+size_t artk_lora_linear_multi_fwd_workspace_bytes(int64_t T, int64_t in, const artk_lora_proj_t* proj,
+                                                  int32_t n);
+int32_t artk_lora_linear_multi_fwd(const void* x, const artk_lora_proj_t* proj, int32_t n, float scale,
+                                   int64_t T, int64_t in, void* workspace, size_t workspace_bytes,
+                                   artk_stream_t stream);
+size_t artk_lora_linear_multi_bwd_workspace_bytes(int64_t T, int64_t in, const artk_lora_proj_t* proj,
+                                                  int32_t n);
+int32_t artk_lora_linear_multi_bwd(const void* x, const artk_lora_proj_t* proj, int32_t n, float scale,
+                                   int64_t T, int64_t in, void* dx, void* workspace, size_t workspace_bytes,
+                                   artk_stream_t stream);
+
+/* ------------------------------------------------------------------------- *
  * Per-kernel timing (measurement aid; no counterpart in the reference).
  * artk_profile_enable(1) makes later calls bracket each dominant kernel with
  * HIP events on the launch stream; after the caller has synchronised,
@@ -408,12 +457,24 @@ int32_t artk_profile_collect(int32_t kind, double* total_ms, int64_t* launches);
  * artk_mfma_loop16: the same arguments and the same work per round as 64 MFMA
  *   16x16x32 instructions on 8 x 4 tiles of 16 x 16 per wave.
  * artk_stream_copy: dst[i] = src[i], 16 bytes per lane and step (bytes % 16 == 0).
+ * artk_lds_probe: LDS bytes per clock of a CU.  `blocks` work-groups of `waves` (4 or 8)
+ *   wavefronts; every wave issues `iters` rounds of 16 LDS reads whose results nothing
+ *   consumes: kind 0 = ds_read_b128, 1 KiB contiguous per wave instruction; kind 1 =
+ *   ds_read_b128 in the swizzled operand-fragment pattern of the GEMM main loop; kind 2 =
+ *   ds_read_b64_tr_b16 (transposed read, 512 bytes per wave instruction).  reads_per_dma
+ *   0: reads only; 2 or 3: one 1 KiB `buffer_load ... lds` write from `src` (64 KiB,
+ *   16-byte aligned, stays in L2) into another part of LDS per that many reads, the mix
+ *   of the 4-wave / 8-wave main loop.  cycles int64 [blocks][2] receives the core-clock
+ *   cycles and the 100 MHz ticks each work-group spent in the loop (barrier to barrier); bytes read
+ *   per work-group: waves * iters * 16 * (1024 | 512).
  * ------------------------------------------------------------------------- */
 int32_t artk_mfma_loop(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
                        float* sink, artk_stream_t stream);
 int32_t artk_mfma_loop16(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
                          float* sink, artk_stream_t stream);
 int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_t stream);
+int32_t artk_lds_probe(int32_t waves, int32_t kind, int32_t reads_per_dma, const void* src, int64_t iters,
+                       int32_t blocks, int64_t* cycles, artk_stream_t stream);
 
 #ifdef __cplusplus
 }

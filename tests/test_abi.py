@@ -24,7 +24,7 @@ def test_header_symbols_are_exported_and_bound(artk_lib):
     for n in names:
         assert hasattr(artk_lib, n), f"{n} declared in artk.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
-    assert artk_lib.artk_abi_version() == 3
+    assert artk_lib.artk_abi_version() == 4
 
 
 def test_argument_errors_have_codes_and_messages(artk_lib):
@@ -47,6 +47,16 @@ def test_argument_errors_have_codes_and_messages(artk_lib):
     assert rc == _lib.ERR_INVALID_ARGUMENT  # clip_lo > clip_hi
     rc = artk_lib.artk_lora_linear_fwd(p, p, p, p, None, 2.0, 64, 64, 64, 5, p, p, p, 4096, None)  # rank 5
     assert rc == _lib.ERR_UNSUPPORTED_SHAPE
+    rc = artk_lib.artk_lora_linear_fwd(p, p, p, p, p + 8, 2.0, 64, 64, 64, 8, p, p, p, 4096, None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"aligned" in artk_lib.artk_last_error()   # misaligned bias
+    projs = (_lib.LoraProjStruct * 5)()
+    rc = artk_lib.artk_lora_linear_multi_fwd(p, projs, 5, 2.0, 64, 64, p, 4096, None)            # five projections
+    assert rc == _lib.ERR_INVALID_ARGUMENT
+    for q in projs:
+        q.W = q.W_t = q.A = q.B = q.y = q.g = q.xa = q.dA = q.dB = p
+        q.out, q.r = 64, 24
+    rc = artk_lib.artk_lora_linear_multi_bwd(p, projs, 3, 2.0, 64, 64, p, p, 1 << 30, None)      # ranks add up to 72
+    assert rc == _lib.ERR_UNSUPPORTED_SHAPE and b"64" in artk_lib.artk_last_error()
     # gathered MoE rows further than 2 GiB from x
     rc = artk_lib.artk_moe_lora_grouped_fwd(p, p, p, p, p, 2.0, p, p, p, 1 << 20, 4096, 64, 8, 8, p, p, p, 4096, None)
     assert rc == _lib.ERR_UNSUPPORTED_SHAPE and b"2 GiB" in artk_lib.artk_last_error()

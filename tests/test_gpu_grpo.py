@@ -131,10 +131,11 @@ def test_fused_wide_logit_range(artk_lib, gpu):
     assert rel_l2(hidden.grad.float().cpu(), ref["d_hidden"]) <= GRAD_TOL
 
 
-def test_fused_target_88_nats_under_the_maximum_is_loud(artk_lib, gpu):
-    """A sampled token whose logit lies more than 88 nats under its row's largest one (probability
-    below e^-88: it cannot have been sampled) overflows the exponential stash: that row's d_hidden is
-    not finite, every other row is unaffected."""
+def test_fused_target_far_under_the_maximum_is_dropped_and_counted(artk_lib, gpu):
+    """A sampled token whose logit lies 95 nats under its row's largest one (probability below
+    e^-80: it cannot have been sampled) would overflow the exponential stash.  That row's d_hidden
+    is written as zeros and counted in metrics["dropped_rows"]; its logprob and the loss stay exact
+    and finite, every other row is unaffected, nothing in d_hidden is inf or NaN."""
     T, H, V = 256, 64, 1024
     hidden = torch.zeros(1, T, H, dtype=torch.bfloat16)
     hidden[0, :, 0] = 1.0
@@ -150,15 +151,49 @@ def test_fused_target_88_nats_under_the_maximum_is_loud(artk_lib, gpu):
     adv = torch.ones(1, T)
     mask = torch.ones(1, T, dtype=torch.bool)
     w = torch.ones(1, T)
-    h = hidden.to(gpu).requires_grad_(True)
-    loss, metrics, logprob = fused_grpo_loss(h, lm_head.to(gpu), tokens.to(gpu), old.to(gpu), adv.to(gpu),
-                                             mask.to(gpu), w.to(gpu))
-    loss.backward()
-    g = h.grad[0].float().cpu()
-    assert abs(logprob[0, 100].item() + 95.0) < 1e-3
-    assert not torch.isfinite(g[100]).all()
-    others = torch.cat([g[:100], g[101:]])
-    assert torch.isfinite(others).all()
+    for skip in (False, True):
+        h = hidden.to(gpu).requires_grad_(True)
+        loss, metrics, logprob = fused_grpo_loss(h, lm_head.to(gpu), tokens.to(gpu), old.to(gpu), adv.to(gpu),
+                                                 mask.to(gpu), w.to(gpu), skip_inactive=skip)
+        loss.backward()
+        g = h.grad[0].float().cpu()
+        assert abs(logprob[0, 100].item() + 95.0) < 1e-3
+        assert torch.isfinite(loss).item() and torch.isfinite(g).all()
+        assert metrics["dropped_rows"].item() == 1.0
+        assert (g[100] == 0).all()
+        # every other row against the oracle (their targets carry all of the probability, so the
+        # rows are tiny: an absolute bound)
+        ref = grpo_oracle.loss_and_grad(hidden, lm_head, tokens, old, adv, mask, w, 0.2, 0.2, chunk_size=T)
+        want = ref["d_hidden"][0]
+        others = torch.cat([torch.arange(100), torch.arange(101, T)])
+        assert (g[others] - want[others]).abs().max().item() <= 1e-6
+        assert abs(loss.item() - ref["loss"].item()) <= LOSS_TOL * abs(ref["loss"].item()) + 2e-6
+
+
+def test_fused_no_grad_runs_the_forward_half_only(artk_lib, gpu):
+    """Under torch.no_grad() (an evaluation pass) the loss comes from the forward kernels alone
+    and equals the training pass's loss and logprobs bit for bit."""
+    T, H, V = 512, 128, 4096
+    case = synthetic.make_grpo_case("t", 98, T, H, V, 4, 4, 0.5)
+    oracle_case(case, 256)   # fills in the old logprobs
+    args = (case.lm_head.to(gpu), case.tokens.to(gpu), case.logprobs.to(gpu), case.advantages.to(gpu),
+            case.assistant_mask.to(gpu), case.weights.to(gpu))
+    h = case.hidden.to(gpu).requires_grad_(True)
+    loss, metrics, logprob = fused_grpo_loss(h, *args)
+    from art_amd import ops
+    ops.profile_enable(True)
+    with torch.no_grad():
+        loss2, metrics2, logprob2 = fused_grpo_loss(h, *args)
+    torch.cuda.synchronize()
+    _, n_bwd = ops.profile_collect(ops.PROF_DHIDDEN_GEMM)
+    _, n_fwd = ops.profile_collect(ops.PROF_LMHEAD_FWD)
+    ops.profile_enable(False)
+    assert n_fwd >= 1 and n_bwd == 0
+    assert loss2.item() == loss.item()
+    assert torch.equal(logprob2, logprob)
+    assert metrics2["policy_loss"].item() == metrics["policy_loss"].item()
+    assert metrics2["dropped_rows"].item() == 0.0
+    assert not loss2.requires_grad
 
 
 def test_unfused_autograd_matches_oracle(artk_lib, gpu):

@@ -181,3 +181,101 @@ def test_lora_module_with_bias_from_linear(artk_lib, gpu):
             + mod.scaling * (x.detach().float() @ mod.lora_A.float().t()) @ mod.lora_B.float().t())
     assert rel_l2(y.detach().float().cpu(), want.cpu()) <= TOL
     assert mod.bias.grad is None and mod.lora_A.grad is not None
+
+
+# ---- projections of the same input in one call (q|k|v, gate|up) ------------------------------------
+_oracle_cache = {}
+
+
+def shared_input_case(T, n_in, outs, ranks, seed, with_bias):
+    """Per projection (W, A, B, bias, g) on one x, and the oracle's (y, dx, dA, dB) of each."""
+    key = (T, n_in, tuple(outs), tuple(ranks), seed, with_bias)
+    if key not in _oracle_cache:
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(T, n_in, generator=g).to(torch.bfloat16)
+        parts, refs = [], []
+        for o, r in zip(outs, ranks):
+            W = (0.02 * torch.randn(o, n_in, generator=g)).to(torch.bfloat16)
+            A = ((torch.rand(r, n_in, generator=g) * 2 - 1) / math.sqrt(n_in)).to(torch.bfloat16)
+            B = (0.01 * torch.randn(o, r, generator=g)).to(torch.bfloat16)
+            bias = (0.5 * torch.randn(o, generator=g)).to(torch.bfloat16) if with_bias else None
+            up = torch.randn(T, o, generator=g).to(torch.bfloat16)
+            parts.append((W, A, B, bias, up))
+        scale = 16 / ranks[0]
+        for W, A, B, bias, up in parts:
+            y0, dx0, dA0, dB0 = lora_oracle.lora_linear_grads(x, W, A, B, scale, up)
+            refs.append((y0 + bias.float() if with_bias else y0, dx0, dA0, dB0))
+        _oracle_cache.clear()          # one case at a time: a gate|up case holds 3 GB of fp32 references
+        _oracle_cache[key] = (x, parts, refs, scale)
+    return _oracle_cache[key]
+
+
+MULTI_CASES = [
+    pytest.param(8192, 2048, (2048, 256, 256), (8, 8, 8), True, id="c2-qkv"),
+    pytest.param(8192, 2048, (11008, 11008), (8, 8), False, id="c2-gate_up"),
+    pytest.param(300, 192, (320, 64), (16, 16), True, id="ragged"),
+    pytest.param(1000, 448, (192, 576, 64, 128), (8, 8, 8, 8), False, id="four"),
+]
+
+
+@pytest.mark.parametrize("T,n_in,outs,ranks,with_bias", MULTI_CASES)
+def test_multi_projection_matches_oracle(artk_lib, gpu, T, n_in, outs, ranks, with_bias):
+    """artk_lora_linear_multi_fwd / _bwd (separate weights, adapters, outputs and upstream gradients)
+    against the oracle evaluated projection by projection; dx is the sum over the projections.  The
+    two config-2 cases are the call shapes of a Qwen2.5-3B layer at full size."""
+    print(f"lora multi T={T} in={n_in} outs={outs} ranks={ranks}", flush=True)
+    x, parts, refs, scale = shared_input_case(T, n_in, outs, ranks, 4242 + T, with_bias)
+    xd = x.to(gpu)
+    Ws = [p[0].to(gpu) for p in parts]
+    As = [p[1].to(gpu) for p in parts]
+    Bs = [p[2].to(gpu) for p in parts]
+    biases = [p[3].to(gpu) for p in parts] if with_bias else None
+    gs = [p[4].to(gpu) for p in parts]
+    ys, xas = ops.lora_linear_multi_fwd(xd, Ws, As, Bs, scale, biases)
+    dx, dAs, dBs = ops.lora_linear_multi_bwd(gs, xd, [ops.transpose(w) for w in Ws], As, Bs, xas, scale)
+    dx0 = sum(r[1] for r in refs)
+    assert rel_l2(dx.cpu().float(), dx0) <= TOL
+    for i, (y0, _, dA0, dB0) in enumerate(refs):
+        assert rel_l2(ys[i].cpu().float(), y0) <= TOL, i
+        assert rel_l2(dAs[i].cpu(), dA0) <= TOL, i
+        assert rel_l2(dBs[i].cpu(), dB0) <= TOL, i
+    # bit-reproducible run to run, and identical to the single-projection entry points on each projection's
+    # own outputs (same kernels and summation orders; dx differs: it is one accumulation here)
+    dx2, dAs2, dBs2 = ops.lora_linear_multi_bwd(gs, xd, [ops.transpose(w) for w in Ws], As, Bs, xas, scale)
+    assert torch.equal(dx, dx2) and all(torch.equal(a, b) for a, b in zip(dAs + dBs, dAs2 + dBs2))
+    y_one, xa_one = ops.lora_linear_fwd(xd, Ws[-1], As[-1], Bs[-1], scale, None if biases is None else biases[-1])
+    assert torch.equal(y_one, ys[-1]) and torch.equal(xa_one, xas[-1])
+
+
+@pytest.mark.parametrize("T,n_in,outs,ranks,with_bias", MULTI_CASES[:2])
+def test_concatenated_projections_config2_full_size(artk_lib, gpu, T, n_in, outs, ranks, with_bias):
+    """The single-projection entry points on the concatenated form of the same cases: weights stacked
+    along the output dimension, A stacked, B block-diagonal (out 2560 / rank 24 with the q, k, v biases;
+    out 22016 / rank 16).  The diagonal blocks of dB are the adapters' gradients; the off-diagonal
+    blocks are derivatives with respect to entries that are pinned to zero and belong to no adapter
+    (they are not zero; they are checked against the oracle's full product like the rest)."""
+    print(f"lora concatenated out={sum(outs)} r={sum(ranks)}", flush=True)
+    x, parts, refs, scale = shared_input_case(T, n_in, outs, ranks, 4242 + T, with_bias)
+    W = torch.cat([p[0] for p in parts], 0)
+    A = torch.cat([p[1] for p in parts], 0)
+    B = torch.zeros(sum(outs), sum(ranks), dtype=torch.bfloat16)
+    o0 = r0 = 0
+    for (p, o, r) in zip(parts, outs, ranks):
+        B[o0:o0 + o, r0:r0 + r] = p[2]
+        o0, r0 = o0 + o, r0 + r
+    bias = torch.cat([p[3] for p in parts]) if with_bias else None
+    up = torch.cat([p[4] for p in parts], 1)
+    xd, Wd, Ad, Bd, upd = (t.to(gpu).contiguous() for t in (x, W, A, B, up))
+    y, xa = ops.lora_linear_fwd(xd, Wd, Ad, Bd, scale, None if bias is None else bias.to(gpu))
+    dx, dA, dB = ops.lora_linear_bwd(upd, xd, ops.transpose(Wd), Ad, Bd, xa, scale)
+    assert rel_l2(dx.cpu().float(), sum(r[1] for r in refs)) <= TOL
+    o0 = r0 = 0
+    for (y0, _, dA0, dB0), o, r in zip(refs, outs, ranks):
+        assert rel_l2(y[:, o0:o0 + o].cpu().float(), y0) <= TOL
+        assert rel_l2(dA[r0:r0 + r].cpu(), dA0) <= TOL
+        assert rel_l2(dB[o0:o0 + o, r0:r0 + r].cpu(), dB0) <= TOL
+        o0, r0 = o0 + o, r0 + r
+    # the whole dB, off-diagonal blocks included: s g^T (x A_cat^T) in fp64 on the CPU
+    xa0 = x.double() @ A.double().t()
+    dB_full = scale * (up.double().t() @ xa0)
+    assert rel_l2(dB.cpu(), dB_full) <= TOL

@@ -69,3 +69,14 @@ def test_stream_copy_is_a_copy(artk_lib, gpu):
     dst = torch.zeros_like(src)
     assert ops.stream_copy(src, dst) == src.numel() * 4
     assert torch.equal(src, dst)
+
+
+@pytest.mark.parametrize("waves,kind,rpd", [(8, 0, 0), (4, 1, 2), (8, 2, 3)])
+def test_lds_probe_reports_a_plausible_rate(artk_lib, gpu, waves, kind, rpd):
+    print(f"lds_probe waves={waves} kind={kind} rpd={rpd}", flush=True)
+    r = ops.lds_probe(waves, kind, rpd, 200, 4, gpu)
+    # a CU cannot read more than a few hundred bytes per clock from LDS, nor fewer than a few
+    assert 8.0 < r["read_B_per_clk"] < 1024.0, r
+    assert (r["dma_write_B_per_clk"] > 0) == (rpd > 0)
+    with pytest.raises(ValueError):
+        ops.lds_probe(3, 0, 0, 1, 1, gpu)

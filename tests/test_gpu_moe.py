@@ -222,6 +222,46 @@ def test_config5_down_projection_full_size(artk_lib, gpu):
         assert rel_l2(dA[e].cpu(), dA0[e]) <= TOL and rel_l2(dB[e].cpu(), dB0[e]) <= TOL
 
 
+def test_config5_fused_gate_up_full_size(artk_lib, gpu):
+    """Benchmark config 5 the way art_amd.moe.MoELoRAExperts runs gate and up: ONE grouped product
+    [128, 1536, 2048] over the gathered token rows, adapters stacked to rank 16 with a block-diagonal
+    B per expert.  y, dx (summed per token), dA and dB against the oracle, also expert by expert;
+    gate and up halves against the oracle of each projection alone."""
+    print("moe config5 fused gate|up", flush=True)
+    T, H, I, E, k, r = 8192, 2048, 768, 128, 8, 8
+    g = torch.Generator().manual_seed(1005)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=g)
+    rt, ref = check_routing(logits, k, gpu)
+    Wg, Ag, Bg = make_experts(E, I, H, r, 1005)
+    Wu, Au, Bu = make_experts(E, I, H, r, 3005)
+    W = torch.cat([Wg, Wu], 1).contiguous()
+    A = torch.cat([Ag, Au], 1).contiguous()
+    B = torch.zeros(E, 2 * I, 2 * r, dtype=torch.bfloat16)
+    B[:, :I, :r], B[:, I:, r:] = Bg, Bu
+    up = torch.randn(T * k, 2 * I, generator=g).to(torch.bfloat16)
+    y0, dx0, dA0, dB0 = moe_oracle.grouped_lora_grads(x, ref["row_token"], W, A, B, 2.0, ref["offsets"], up)
+    y, xa = ops.moe_lora_grouped_fwd(x.to(gpu), rt.row_token, W.to(gpu), A.to(gpu), B.to(gpu), 2.0, rt)
+    dx, dA, dB = ops.moe_lora_grouped_bwd(up.to(gpu), x.to(gpu), rt.row_token, ops.transpose_batched(W.to(gpu)),
+                                          A.to(gpu), B.to(gpu), xa, 2.0, rt)
+    dx = dx[rt.inv_perm.long()].view(T, k, H).float().sum(1)
+    assert rel_l2(y.cpu().float(), y0) <= TOL
+    assert rel_l2(dx.cpu(), dx0) <= TOL
+    assert rel_l2(dA.cpu(), dA0) <= TOL
+    assert rel_l2(dB.cpu(), dB0) <= TOL
+    off = ref["offsets"].tolist()
+    for e in (0, 1, 63, 127):
+        sl = slice(off[e], off[e + 1])
+        assert rel_l2(y[sl].cpu().float(), y0[sl]) <= TOL
+        assert rel_l2(dA[e].cpu(), dA0[e]) <= TOL and rel_l2(dB[e].cpu(), dB0[e]) <= TOL
+    # the halves are the two projections: forward and adapter gradients of gate alone
+    yg0, _, dAg0, dBg0 = moe_oracle.grouped_lora_grads(x, ref["row_token"], Wg, Ag, Bg, 2.0, ref["offsets"],
+                                                        up[:, :I].contiguous())
+    assert rel_l2(y[:, :I].cpu().float(), yg0) <= TOL
+    assert rel_l2(dA[:, :r].cpu(), dAg0) <= TOL
+    assert rel_l2(dB[:, :I, :r].cpu(), dBg0) <= TOL
+
+
 def test_moe_block_autograd(artk_lib, gpu):
     """The whole block (gate, up, SiLU gating, down, recombination) against torch fp32."""
     torch.manual_seed(0)
