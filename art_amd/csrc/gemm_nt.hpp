@@ -57,15 +57,21 @@ struct OperandLoader {
   static constexpr int DI = 2 * NI;
   __amdgpu_buffer_rsrc_t rsrc;
   int voff[DI];  // per-lane byte offset of the DMA instructions of this wave
+  int nlive;     // DMA instructions of this wave that are issued (wave-uniform): DI, or, with
+                 // skip_dead, those that carry at least one row of the operand
 
   // base: first element of the operand; ld: leading dimension in elements;
   // row0: first tile row; nrows: rows the operand really has (rows past the
   // end are clamped to the last valid row; the epilogue never stores them).
   // gather (optional): tile row i reads operand row gather[row0 + i] instead of
   // row0 + i; all gathered rows must lie within 2 GiB of `base`.
+  // skip_dead: instructions whose 8 rows all lie past the end are not issued at all; their LDS
+  // rows keep whatever an earlier tile left there, so the accumulator columns (or rows) they
+  // feed hold garbage, possibly NaN, and the caller must discard them (a partial tile's
+  // epilogue does not store them anyway; garbage in one operand row never reaches another).
   __device__ __forceinline__ void init(const void* base, int64_t ld, int64_t row0,
                                        int64_t nrows, int wave, int lane,
-                                       const int* gather = nullptr) {
+                                       const int* gather = nullptr, bool skip_dead = false) {
     const char* p = (const char*)base + (gather ? 0 : row0 * ld * 2);
     rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
     int64_t left = nrows - row0;
@@ -79,21 +85,29 @@ struct OperandLoader {
       if (gather) rc = gather[row0 + rc];
       voff[i] = (int)(rc * ld * 2) + kc * 16;
     }
+    nlive = DI;
+    if (skip_dead) {
+      const int live = (nvalid + 7) / 8 - wave * DI;  // instruction j of the tile carries rows 8j .. 8j+7
+      nlive = live < 0 ? 0 : (live < DI ? live : DI);
+    }
   }
 
   // Issue DMA instructions LO..HI-1 of this wave's DI for K offset k0 (elements)
   // into the 32 KiB operand stage at `stage` (LDS byte address, wave-uniform).
   // DMA instruction i alone (i a compile-time constant at every call site).
   __device__ __forceinline__ void issue_one(char* stage, int wave, int k0, int i) const {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * DI + i) * 1024), 16, voff[i],
-                                             k0 * 2, 0, 0);
+    if (i < nlive)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * DI + i) * 1024), 16, voff[i],
+                                               k0 * 2, 0, 0);
   }
-  template <int LO, int HI>
+  // (TAG is unused: callers that are themselves instantiated several times pass a distinct value each)
+  template <int LO, int HI, int TAG = 0>
   __device__ __forceinline__ void issue(char* stage, int wave, int k0) const {
 #pragma unroll
     for (int i = LO; i < HI; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * DI + i) * 1024), 16,
-                                               voff[i], k0 * 2, 0, 0);
+      if (i < nlive)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(stage + (wave * DI + i) * 1024), 16,
+                                                 voff[i], k0 * 2, 0, 0);
     }
   }
 };
@@ -128,20 +142,24 @@ struct Frags {
   bf16x8 p[4], q[NI];
 };
 
-template <int NI>
+// NQ (<= NI): column-operand tiles of this wave that are computed; the others are left alone
+// (a partial tile whose last columns nobody stores).  NQ = 0: nothing is read or multiplied.
+template <int NI, int NQ = NI>
 __device__ __forceinline__ void load_frags(Frags<NI>& f, const char* sp, const char* sq, int off) {
+  if constexpr (NQ > 0) {
 #pragma unroll
-  for (int mi = 0; mi < 4; ++mi) f.p[mi] = *(const bf16x8*)(sp + off + mi * 4096);
+    for (int mi = 0; mi < 4; ++mi) f.p[mi] = *(const bf16x8*)(sp + off + mi * 4096);
 #pragma unroll
-  for (int ni = 0; ni < NI; ++ni) f.q[ni] = *(const bf16x8*)(sq + off + ni * 4096);
+    for (int ni = 0; ni < NQ; ++ni) f.q[ni] = *(const bf16x8*)(sq + off + ni * 4096);
+  }
 }
 
-template <int NI>
+template <int NI, int NQ = NI>
 __device__ __forceinline__ void mma_frags(TileAcc<NI>& acc, const Frags<NI>& f) {
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
+    for (int ni = 0; ni < NQ; ++ni)
       acc.c[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.p[mi], f.q[ni], acc.c[mi][ni], 0, 0, 0);
 }
 
@@ -181,11 +199,11 @@ struct TileLoaders {
   int k_begin, k_end;
   __device__ __forceinline__ void init(const void* P, int64_t ldp, int64_t prow0, int64_t prows,
                                        const void* Q, int64_t ldq, int64_t qrow0, int64_t qrows, int kb,
-                                       int ke, const int* qgather = nullptr) {
+                                       int ke, const int* qgather = nullptr, bool q_skip_dead = false) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     lp.init(P, ldp, prow0, prows, wave, lane);
-    lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather);
+    lq.init(Q, ldq, qrow0, qrows, wave, lane, qgather, q_skip_dead);
     k_begin = kb;
     k_end = ke;
   }
@@ -215,7 +233,7 @@ struct TileLoaders {
 // that would reach past the end of the K range.
 __device__ __forceinline__ void gemm_tile_run_pinned(TileAcc<4>& acc, char* smem, const TileLoaders<4>& L);
 
-template <int NI>
+template <int NI, int NQ = NI>
 __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const TileLoaders<NI>& L) {
   if constexpr (NI == 4) {
     gemm_tile_run_pinned(acc, smem, L);  // one wave per SIMD: the order is pinned (see below)
@@ -247,11 +265,11 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (nk > 1) {
-    lp.template issue<0, EARLY>(smem + STAGE_BYTES, wave, k_begin + BK);
-    lq.template issue<0, EARLY>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
+    lp.template issue<0, EARLY, NQ>(smem + STAGE_BYTES, wave, k_begin + BK);
+    lq.template issue<0, EARLY, NQ>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
   }
   Frags<NI> f0, f1;
-  load_frags(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
+  load_frags<NI, NQ>(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
 
   // One K-step.  LATE: the second half of stage kt + 1 is still to be issued (false in the last
   // K-step); AHEAD: the first half of stage kt + 2 goes out after the barrier (false in the last
@@ -266,15 +284,15 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (LATE) {
       const int k1 = k_begin + (kt + 1) * BK;
-      lp.template issue<EARLY, DI>(nxt, wave, k1);
-      lq.template issue<EARLY, DI>(nxt + OPER_STAGE_BYTES, wave, k1);
+      lp.template issue<EARLY, DI, NQ>(nxt, wave, k1);
+      lq.template issue<EARLY, DI, NQ>(nxt + OPER_STAGE_BYTES, wave, k1);
     }
-    load_frags(f1, sp, sq, off[1]);
-    mma_frags(acc, f0);
-    load_frags(f0, sp, sq, off[2]);
-    mma_frags(acc, f1);
-    load_frags(f1, sp, sq, off[3]);
-    mma_frags(acc, f0);
+    load_frags<NI, NQ>(f1, sp, sq, off[1]);
+    mma_frags<NI, NQ>(acc, f0);
+    load_frags<NI, NQ>(f0, sp, sq, off[2]);
+    mma_frags<NI, NQ>(acc, f1);
+    load_frags<NI, NQ>(f1, sp, sq, off[3]);
+    mma_frags<NI, NQ>(acc, f0);
     // Interleave: 3 steps of 4*NI MFMAs, 3*(4+NI) LDS reads, 2*(DI-EARLY) DMA issues.
     constexpr int NLATE = LATE ? 2 * (DI - EARLY) : 0;
     if constexpr (NI == 4) {
@@ -309,12 +327,12 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (AHEAD) {
       const int k2 = k_begin + (kt + 2) * BK;
-      lp.template issue<0, EARLY>(cur, wave, k2);
-      lq.template issue<0, EARLY>(cur + OPER_STAGE_BYTES, wave, k2);
+      lp.template issue<0, EARLY, NQ>(cur, wave, k2);
+      lq.template issue<0, EARLY, NQ>(cur + OPER_STAGE_BYTES, wave, k2);
     }
     // (after the last K-step this reads the idle stage: values nobody uses)
-    load_frags(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
-    mma_frags(acc, f1);
+    load_frags<NI, NQ>(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
+    mma_frags<NI, NQ>(acc, f1);
     // 4*NI MFMA, 4+NI LDS reads, 2*EARLY DMA issues
     if constexpr (NI == 4) {
 #pragma unroll
@@ -341,6 +359,18 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
   // Nothing is outstanding here; the caller may reuse or release LDS.
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
+}
+
+// gemm_tile_run for a tile whose column operand has only `ncols` (<= 256) rows that anybody
+// stores: a wave computes only those of its NI 32-column tiles that contain such a column
+// (wave-uniform choice; every variant executes the same barriers).  8-wave shape only.
+__device__ __forceinline__ void gemm_tile_run_cols(TileAcc<2>& acc, char* smem, const TileLoaders<2>& L,
+                                                   int ncols) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int left = ncols - wave_n<2>(wave) * 64;  // columns of this wave that are stored
+  if (left > 32) gemm_tile_run<2, 2>(acc, smem, L);
+  else if (left > 0) gemm_tile_run<2, 1>(acc, smem, L);
+  else gemm_tile_run<2, 0>(acc, smem, L);
 }
 
 // ----------------------------------------------------------------------------

@@ -270,8 +270,9 @@ __device__ __forceinline__ MoeTile moe_tile(const MoeGemmParams& p, int t, int n
 
 __device__ __forceinline__ void moe_tile_loaders(TileLoaders<MOE_NI>& L, const MoeGemmParams& p,
                                                  const MoeTile& m) {
+  // rows past the expert's end are not fetched (their output columns are never stored)
   L.init((const char*)p.W + (int64_t)m.e * p.M * p.K * 2, p.K, (int64_t)m.mt * TILE, p.M, p.X, p.K, m.row0,
-         m.row_end, 0, (int)p.K, p.gather);
+         m.row_end, 0, (int)p.K, p.gather, true);
 }
 
 // Persistent work-groups: tiles t, t + grid, ... of the device-side work list; the
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(nthreads<MOE_NI>()) void moe_gemm_kernel(MoeGemmPar
     {
       TileLoaders<MOE_NI> L;  // its first stage is already on the way
       moe_tile_loaders(L, p, cur);
-      gemm_tile_run(acc, smem, L);
+      gemm_tile_run_cols(acc, smem, L, cur.nvalid);  // a tail tile computes only its live 32-row blocks
     }
     if (more) {
       TileLoaders<MOE_NI> L;

@@ -512,18 +512,53 @@ def bench_moe(args):
                                            "note": "softmax/top-k/stable sort + per-expert F.linear loop with "
                                                    "autograd, bf16, same three projections"}
     if not args.no_cpu_baseline:
+        import hashlib
+
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         import moe_oracle
 
-        t0 = time.perf_counter()
-        ref = moe_oracle.route(logits.cpu(), k)
-        moe_oracle.grouped_lora_grads(x.cpu(), ref["row_token"], Wg.cpu(), Ag.cpu(), Bg.cpu(), scale,
-                                      ref["offsets"], g_i.cpu())
-        cdt = time.perf_counter() - t0
-        one = 2 * 2.0 * n * H * I + 6.0 * n * r * (H + I)
-        res["cpu_baseline"] = {"value": one / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+        # CPU oracle (fp32) of routing and all three projections (gate, up over the gathered token rows,
+        # down over the sorted rows): the timing sample, 1 warm-up + 3 runs, median
+        cpu_in = {"gate": (x.cpu(), True, Wg.cpu(), Ag.cpu(), Bg.cpu(), g_i.cpu()),
+                  "up": (x.cpu(), True, Wu.cpu(), Au.cpu(), Bu.cpu(), g_i.cpu()),
+                  "down": (h.cpu(), False, Wd.cpu(), Ad.cpu(), Bd.cpu(), g_h.cpu())}
+        times, ref, ref_out = [], None, {}
+        for rep in range(4):
+            t0 = time.perf_counter()
+            ref = moe_oracle.route(logits.cpu(), k)
+            for name, (xin, gathered, W_, A_, B_, up_) in cpu_in.items():
+                out = moe_oracle.grouped_lora_grads(xin, ref["row_token"] if gathered else None, W_, A_, B_, scale,
+                                                    ref["offsets"], up_)
+                if rep == 0:
+                    ref_out[name] = out
+            if rep:
+                times.append(time.perf_counter() - t0)
+        cdt = sorted(times)[1]
+        res["cpu_baseline"] = {"value": flops / cdt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
                                "kind": "port",
-                               "sample": f"routing + gate projection fwd+bwd, fp32 torch-CPU oracle, 1 run of {cdt:.1f} s"}
+                               "sample": f"routing + gate, up and down projections fwd+bwd, fp32 torch-CPU oracle, "
+                                         f"1 warm-up + 3 runs, median {cdt:.1f} s"}
+        # parity of this run: integer outputs of the routing by digest, the fused gate|up product (the
+        # measured path) and the down product by rel-L2 against the oracle of each projection
+        sha = lambda t: hashlib.sha256(t.cpu().to(torch.int64).contiguous().numpy().tobytes()).hexdigest()
+        rt = ops.moe_route(logits, k)
+        ints = {}
+        for key in ("topk_idx", "perm", "inv_perm", "row_token", "offsets"):
+            ints[key] = {"sha256": sha(getattr(rt, key))[:16], "equal": sha(getattr(rt, key)) == sha(ref[key])}
+        rel = lambda a, b: ((a.double().cpu() - b.double()).norm() / b.double().norm()).item()
+        ygu, xagu = ops.moe_lora_grouped_fwd(x, rt.row_token, Wgu, Agu, Bgu, scale, rt)
+        dxr, dAgu, dBgu = ops.moe_lora_grouped_bwd(g_i2, x, rt.row_token, Wgut, Agu, Bgu, xagu, scale, rt)
+        dx_tok = dxr[rt.inv_perm.long()].view(T, k, H).float().sum(1)
+        yg0, dxg0, dAg0, dBg0 = ref_out["gate"]
+        yu0, dxu0, dAu0, dBu0 = ref_out["up"]
+        fused = {"y_gate": rel(ygu[:, :I], yg0), "y_up": rel(ygu[:, I:], yu0), "dx": rel(dx_tok, dxg0 + dxu0),
+                 "dA_gate": rel(dAgu[:, :r], dAg0), "dA_up": rel(dAgu[:, r:], dAu0),
+                 "dB_gate": rel(dBgu[:, :I, :r], dBg0), "dB_up": rel(dBgu[:, I:, r:], dBu0)}
+        yd, xad = ops.moe_lora_grouped_fwd(h, None, Wd, Ad, Bd, scale, rt)
+        dxd, dAd, dBd = ops.moe_lora_grouped_bwd(g_h, h, None, Wdt, Ad, Bd, xad, scale, rt)
+        down = dict(zip(("y", "dx", "dA", "dB"), (rel(a, b) for a, b in zip((yd, dxd, dAd, dBd), ref_out["down"]))))
+        res["parity_same_run"] = {"routing_bit_exact": ints, "fused_gate_up": fused, "down": down,
+                                  "tolerance_rel_l2": 1e-2}
     return res
 
 
