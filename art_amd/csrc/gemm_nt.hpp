@@ -532,15 +532,25 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
 
 
 // Logical tile id -> (row-operand tile, column-operand tile).  Ids walk down a
-// group of GROUP row-operand tiles before moving to the next column-operand
-// tile, so the 32 work-groups that run together on one XCD cover a GROUP x
-// (32/GROUP) patch and share operand panels in that XCD's L2.
+// group of `group` row-operand tiles before moving to the next column-operand
+// tile, so the 32 work-groups that run together on one XCD cover a group x
+// (32/group) patch and share operand panels in that XCD's L2.  Which split of the
+// 32 is best depends on where the operands come from: a patch fetches `group`
+// row-operand panels and 32/group column-operand panels per K step, and a panel of
+// a small operand that every XCD keeps re-reading (the hidden states of a chunk,
+// the activations of a layer) is served by the Infinity Cache, while the panels of
+// a large streaming operand (the 1.1 GB lm_head) come from HBM the first time.
+// Measured on 152064 x 5632 x 3584 (lm_head forward): group 4 gives 1290 TFLOP/s,
+// 3 / 5 / 6: 1255, 8: 1222, 2: 1240, 16: 1105; on 22016 x 8192 x 2048 (LoRA
+// gate|up, both operands resident): 8 gives 1225, 4 and 16: 1160, 2: 1070.
 constexpr int TILE_GROUP = 8;
-__device__ __forceinline__ void tile_coords(int id, int row_tiles, int col_tiles, int& rt, int& ct) {
-  const int per = TILE_GROUP * col_tiles;
+constexpr int TILE_GROUP_STREAMING = 4;  // row operand streams from HBM, column operand is small
+__device__ __forceinline__ void tile_coords(int id, int row_tiles, int col_tiles, int& rt, int& ct,
+                                            int group = TILE_GROUP) {
+  const int per = group * col_tiles;
   const int g = id / per;
-  const int first = g * TILE_GROUP;
-  const int gs = row_tiles - first < TILE_GROUP ? row_tiles - first : TILE_GROUP;
+  const int first = g * group;
+  const int gs = row_tiles - first < group ? row_tiles - first : group;
   const int w = id - g * per;
   rt = first + w % gs;
   ct = w / gs;

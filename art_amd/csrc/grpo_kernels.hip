@@ -194,7 +194,7 @@ __device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, 
 __device__ __forceinline__ bool lmhead_next_tile(const FwdParams& p, int n_tiles, int n, int& t, int& vt,
                                                  int& tt) {
   for (; t < n_tiles; t += gridDim.x) {
-    tile_coords(xcd_remap(t, n_tiles), p.VT, p.TT, vt, tt);
+    tile_coords(xcd_remap(t, n_tiles), p.VT, p.TT, vt, tt, TILE_GROUP_STREAMING);
     if (tt * TILE < n) return true;
   }
   return false;
@@ -779,7 +779,7 @@ __global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   int mt, nt;
-  tile_coords(id, p.MT, p.NT, mt, nt);
+  tile_coords(id, p.MT, p.NT, mt, nt, p.MT >= 8 * p.NT ? TILE_GROUP_STREAMING : TILE_GROUP);
   TileAcc<GEMM_NI> acc;
   acc.zero();
   gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,

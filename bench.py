@@ -1070,7 +1070,7 @@ def main():
 
     chunk = args.chunk_tokens or ops.DEFAULT_CHUNK_TOKENS  # 0 = library default
     ws = torch.empty(ops.grpo_fused_workspace_bytes(T, V, H, chunk), dtype=torch.uint8, device=dev)
-    out = (torch.empty(4, dtype=torch.float32, device=dev),
+    out = (torch.empty(5, dtype=torch.float32, device=dev),
            torch.empty(T, dtype=torch.float32, device=dev),
            torch.empty((T, H), dtype=torch.bfloat16, device=dev))
 
