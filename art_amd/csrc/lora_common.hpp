@@ -95,8 +95,7 @@ struct SmallTranspose {
   uint16_t* dst;
   int64_t n, R, C;  // n matrices of [R, C]
 };
-__global__ __launch_bounds__(256) static void small_transpose2_kernel(SmallTranspose a, SmallTranspose b) {
-  const SmallTranspose t = blockIdx.y == 0 ? a : b;
+__device__ __forceinline__ void small_transpose_one(const SmallTranspose& t) {
   const int64_t RB = t.R / 8, CB = t.C / 8;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= t.n * RB * CB) return;
@@ -124,6 +123,28 @@ __global__ __launch_bounds__(256) static void small_transpose2_kernel(SmallTrans
     }
     *(uint4*)(dst + c * t.R) = make_uint4(o[0], o[1], o[2], o[3]);
   }
+}
+__global__ __launch_bounds__(256) static void small_transpose2_kernel(SmallTranspose a, SmallTranspose b) {
+  small_transpose_one(blockIdx.y == 0 ? a : b);
+}
+// Up to 8 jobs in one launch (the factors of several projections).
+struct SmallTransposeMulti {
+  SmallTranspose t[8];
+  int n;
+};
+__global__ __launch_bounds__(256) static void small_transpose_multi_kernel(SmallTransposeMulti m) {
+  small_transpose_one(m.t[blockIdx.y]);
+}
+static inline int32_t launch_small_transpose_multi(const SmallTransposeMulti& m, hipStream_t st) {
+  int64_t big = 0;
+  for (int i = 0; i < m.n; ++i) {
+    const int64_t e = m.t[i].n * m.t[i].R * m.t[i].C / 64;  // 8 x 8 blocks
+    big = e > big ? e : big;
+  }
+  dim3 grid((unsigned)((big + 255) / 256), (unsigned)m.n);
+  small_transpose_multi_kernel<<<grid, 256, 0, st>>>(m);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
 }
 
 static inline int32_t launch_small_transpose2(const void* s0, void* d0, int64_t n0, int64_t R0, int64_t C0,

@@ -614,25 +614,49 @@ int32_t artk_lora_linear_multi_bwd(const void* x, const artk_lora_proj_t* proj, 
   p.n_tiles = MT * p.NT;
   StatsReduceJob jx{c.colp_x, c.gx.n_slabs, in, scale, nullptr, 1, nullptr, 0, 0.f};
   jx.n_split = n;
+  SmallTransposeMulti tr;
+  StatsMulti sm;
+  StatsReduceMulti rm;
+  tr.n = 2 * n;
+  sm.n = n;
+  rm.n = 2 * n;
+  bool any_wide = false, any_narrow = false;
   int r0 = 0;
   for (int i = 0; i < n; ++i) {
     const artk_lora_proj_t& q = proj[i];
     LoraBwdScratch& o = c.one[i];
     const int RP = round16(q.r);
-    if ((rc = launch_small_transpose2(q.B, o.Bt, 1, q.out, q.r, q.A, o.At, 1, q.r, in, st))) return rc;
+    (q.r > 32 ? any_wide : any_narrow) = true;
+    tr.t[2 * i] = SmallTranspose{(const uint16_t*)q.B, o.Bt, 1, q.out, q.r};
+    tr.t[2 * i + 1] = SmallTranspose{(const uint16_t*)q.A, o.At, 1, q.r, in};
     // one pass over g_i: partials of g_i B_i (over column chunks) and of g_i^T (x A_i^T) (over row slabs)
-    if ((rc = launch_stats(q.g, T, q.out, o.Bt, q.xa, q.r, o.gg, o.rowp_g, o.colp_g, c.dummy, st))) return rc;
+    sm.p[i] = stats_params(q.g, T, q.out, o.Bt, q.xa, q.r, o.gg, o.rowp_g, o.colp_g, c.dummy);
     StatsReduceJob ja{o.rowp_g, o.gg.n_chunks, T, 1.f, c.gb_cat, 0, o.gb16, RP, scale};
     ja.out_ld = c.r_total;
     ja.out_off = r0;
-    StatsReduceJob jb{o.colp_g, o.gg.n_slabs, q.out, scale, q.dB, 0, nullptr, 0, 0.f};
-    if ((rc = launch_stats_reduce(ja, jb, q.r, st))) return rc;
+    rm.job[2 * i] = ja;
+    rm.job[2 * i + 1] = StatsReduceJob{o.colp_g, o.gg.n_slabs, q.out, scale, q.dB, 0, nullptr, 0, 0.f};
+    rm.R[2 * i] = rm.R[2 * i + 1] = q.r;
     p.seg[i] = LoraSeg{q.W_t, q.g, o.At, o.gb16, q.out, q.r, RP};
     jx.outs[i] = q.dA;
     jx.e_start[i] = r0;
     r0 += q.r;
   }
   jx.e_start[n] = r0;
+  if ((rc = launch_small_transpose_multi(tr, st))) return rc;
+  if (any_wide && any_narrow) {  // the stats kernel has one shape per side of rank 32: one launch per projection
+    for (int i = 0; i < n; ++i) {
+      const StatsParams& sp = sm.p[i];
+      if (sp.R > 32)
+        lora_stats_kernel<2, 2, 2, false><<<(unsigned)(sp.n_slabs * sp.n_chunks), 256, 0, st>>>(sp);
+      else
+        lora_stats_kernel<1, 4, 3, false><<<(unsigned)(sp.n_slabs * sp.n_chunks), 256, 0, st>>>(sp);
+      ARTK_CHECK_LAUNCH();
+    }
+  } else if ((rc = launch_stats_multi(sm, any_wide, st))) {
+    return rc;
+  }
+  if ((rc = launch_stats_reduce_multi(rm, st))) return rc;
   // dx = sum_i ( g_i W_i + (s g_i B_i) A_i ): one launch, the projections as K segments
   if ((rc = launch_lora_multi(p, st))) return rc;
   // one pass over x: [dA_0; dA_1; ...] = s [g_0 B_0 | g_1 B_1 | ...]^T x

@@ -84,7 +84,7 @@ __device__ __forceinline__ bf16x8 st_tr_frag(const char* tile, int lane, int k0,
 // q into a private slot, NST row tiles ahead of the first tile that needs them, ordered
 // (p % 8) 4 + p / 8 so that a lane reads the 8 it needs as two 16-byte LDS loads.
 template <int NTE, int NCT, int NST, bool GATHER>
-__global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
+__device__ __forceinline__ void lora_stats_body(const StatsParams& p, const int block) {
   constexpr int CC = NCT * ST_TILE;
   constexpr int FPITCH = CC + 8;  // halfwords; +16 bytes: rows e land in different banks
   constexpr int YRAW_BYTES = ST_TILE * NTE * 32 * 4;
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int m = lane & 31, half = lane >> 5;
-  const int slab = blockIdx.x / p.n_chunks, chunk = blockIdx.x - slab * p.n_chunks;
+  const int slab = block / p.n_chunks, chunk = block - slab * p.n_chunks;
   const bool grouped = p.offsets != nullptr;
   const int64_t t0 = grouped ? (int64_t)p.offsets[slab] : (int64_t)slab * p.rows_per_slab;
   const int64_t c0 = (int64_t)chunk * p.cc;
@@ -322,6 +322,26 @@ __global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
   }
 }
 
+template <int NTE, int NCT, int NST, bool GATHER>
+__global__ __launch_bounds__(256) void lora_stats_kernel(StatsParams p) {
+  lora_stats_body<NTE, NCT, NST, GATHER>(p, (int)blockIdx.x);
+}
+
+// Several independent passes (the upstream gradients of projections that share an input) in one
+// launch: work-groups block0[i] .. block0[i+1]-1 run pass i.
+constexpr int STATS_MULTI_MAX = 4;
+struct StatsMulti {
+  StatsParams p[STATS_MULTI_MAX];
+  int block0[STATS_MULTI_MAX + 1];
+  int n;
+};
+template <int NTE, int NCT, int NST>
+__global__ __launch_bounds__(256) void lora_stats_multi_kernel(StatsMulti m) {
+  int i = 0;
+  while (i + 1 < m.n && (int)blockIdx.x >= m.block0[i + 1]) ++i;
+  lora_stats_body<NTE, NCT, NST, false>(m.p[i], (int)blockIdx.x - m.block0[i]);
+}
+
 // out[i][e] = scale * sum over parts (fixed order) of part[k][i][e]; written as f32 [n][R] (or
 // [R][n] when transposed) and, optionally, as bf16 [n][RP] times bf16_scale, zero padded to RP.
 struct StatsReduceJob {
@@ -344,10 +364,7 @@ struct StatsReduceJob {
   int e_start[5] = {0, 0, 0, 0, 0};
 };
 
-__global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob a, StatsReduceJob b, int R, int nblk_a) {
-  const bool first = (int)blockIdx.x < nblk_a;
-  const StatsReduceJob j = first ? a : b;
-  const int64_t i = (int64_t)(first ? blockIdx.x : blockIdx.x - nblk_a) * 256 + threadIdx.x;
+__device__ __forceinline__ void stats_reduce_one(const StatsReduceJob& j, int R, int64_t i) {
   const int width = j.out_bf16 ? j.RP : R;
   if (i >= j.n * width) return;
   const int64_t row = i / width;
@@ -378,6 +395,11 @@ __global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob
     }
   }
   if (j.out_bf16) j.out_bf16[row * j.RP + e] = f32_to_bf16(s * j.bf16_scale);
+}
+
+__global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob a, StatsReduceJob b, int R, int nblk_a) {
+  const bool first = (int)blockIdx.x < nblk_a;
+  stats_reduce_one(first ? a : b, R, (int64_t)(first ? blockIdx.x : blockIdx.x - nblk_a) * 256 + threadIdx.x);
 }
 
 struct StatsGeom {
@@ -429,9 +451,8 @@ static inline StatsGeom stats_geom(int64_t T, int64_t C, int r) {
   return best;
 }
 
-static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const uint16_t* F, const float* Y, int r,
-                            const StatsGeom& g, float* row_part, float* col_part, float* row_dummy,
-                            hipStream_t st) {
+static inline StatsParams stats_params(const void* X, int64_t T, int64_t C, const uint16_t* F, const float* Y, int r,
+                                       const StatsGeom& g, float* row_part, float* col_part, float* row_dummy) {
   StatsParams p;
   p.X = (const uint16_t*)X;
   p.T = T;
@@ -452,11 +473,34 @@ static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const ui
   p.n_slabs = g.n_slabs;
   p.n_chunks = g.n_chunks;
   p.cc = g.cc;
+  return p;
+}
+
+static inline int32_t launch_stats(const void* X, int64_t T, int64_t C, const uint16_t* F, const float* Y, int r,
+                            const StatsGeom& g, float* row_part, float* col_part, float* row_dummy,
+                            hipStream_t st) {
+  const StatsParams p = stats_params(X, T, C, F, Y, r, g, row_part, col_part, row_dummy);
   const unsigned grid = (unsigned)(g.n_slabs * g.n_chunks);
   if (r > 32)
     lora_stats_kernel<2, 2, 2, false><<<grid, 256, 0, st>>>(p);
   else
     lora_stats_kernel<1, 4, 3, false><<<grid, 256, 0, st>>>(p);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+// The passes of m in one launch; all ranks on the same side of 32 (the caller checks).
+static inline int32_t launch_stats_multi(StatsMulti& m, bool wide_rank, hipStream_t st) {
+  int blocks = 0;
+  for (int i = 0; i < m.n; ++i) {
+    m.block0[i] = blocks;
+    blocks += m.p[i].n_slabs * m.p[i].n_chunks;
+  }
+  m.block0[m.n] = blocks;
+  if (wide_rank)
+    lora_stats_multi_kernel<2, 2, 2><<<(unsigned)blocks, 256, 0, st>>>(m);
+  else
+    lora_stats_multi_kernel<1, 4, 3><<<(unsigned)blocks, 256, 0, st>>>(m);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }
@@ -528,6 +572,31 @@ static inline int32_t launch_stats_reduce(const StatsReduceJob& a, const StatsRe
   const int64_t na = a.n * (a.out_bf16 ? a.RP : r), nb = b.n * (b.out_bf16 ? b.RP : r);
   const int blk_a = (int)((na + 255) / 256), blk_b = (int)((nb + 255) / 256);
   stats_reduce_kernel<<<(unsigned)(blk_a + blk_b), 256, 0, st>>>(a, b, r, blk_a);
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+// Up to 2 * STATS_MULTI_MAX reductions in one launch; job i reduces partials of rank R[i].
+struct StatsReduceMulti {
+  StatsReduceJob job[2 * STATS_MULTI_MAX];
+  int R[2 * STATS_MULTI_MAX];
+  int block0[2 * STATS_MULTI_MAX + 1];
+  int n;
+};
+__global__ __launch_bounds__(256) static void stats_reduce_multi_kernel(StatsReduceMulti m) {
+  int k = 0;
+  while (k + 1 < m.n && (int)blockIdx.x >= m.block0[k + 1]) ++k;
+  stats_reduce_one(m.job[k], m.R[k], (int64_t)((int)blockIdx.x - m.block0[k]) * 256 + threadIdx.x);
+}
+static inline int32_t launch_stats_reduce_multi(StatsReduceMulti& m, hipStream_t st) {
+  int blocks = 0;
+  for (int i = 0; i < m.n; ++i) {
+    const StatsReduceJob& j = m.job[i];
+    m.block0[i] = blocks;
+    blocks += (int)((j.n * (j.out_bf16 ? j.RP : m.R[i]) + 255) / 256);
+  }
+  m.block0[m.n] = blocks;
+  stats_reduce_multi_kernel<<<(unsigned)blocks, 256, 0, st>>>(m);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

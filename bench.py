@@ -246,17 +246,18 @@ def bench_lora(args):
     groups = (("q", "k", "v"), ("o",), ("gate", "up"))
     fused_mods = [FusedLoRALinear([mods[n] for n in grp]) for grp in groups]
     ups = [[shapes[n][5] for n in grp] for grp in groups]
-    xg = x.detach().requires_grad_(True)
+    # in the model the three groups read three different activations (the attention input, the attention
+    # output, the MLP input): one leaf per group, all with the same values so that one oracle serves
+    xgs = [x.detach().clone().requires_grad_(True) for _ in groups]
     params = [p for m in mods.values() for p in (m.lora_A, m.lora_B)]
     for m in fused_mods:   # transposed copies of the frozen weights are made once per weight version
         for l in m.layers:
             ops.transposed_weight(l.weight)
 
     def step_module():
-        xg.grad = None
-        for p_ in params:
+        for p_ in params + xgs:
             p_.grad = None
-        for m, u in zip(fused_mods, ups):
+        for m, u, xg in zip(fused_mods, ups, xgs):
             torch.autograd.backward(m(xg), u)
 
     def step_raw_multi():
@@ -376,9 +377,11 @@ def bench_lora(args):
                 rec[f"dB_{name}"] = rel(dBs[i], ref[name][3])
             parity["multi_" + "_".join(grp)] = rec
             del ys, dx, dAs, dBs
-        # the module step itself: x.grad is the sum over all six projections
+        # the module step itself: the gradient of each group's input is the sum over its projections
         step_module()
-        rec = {"x_grad": rel(xg.grad, sum(ref[n][1] for n in names))}
+        rec = {}
+        for grp, xg in zip(groups, xgs):
+            rec["x_grad_" + "_".join(grp)] = rel(xg.grad, sum(ref[n][1] for n in grp))
         for name in names:
             rec[f"dA_{name}"] = rel(mods[name].lora_A.grad, ref[name][2])
             rec[f"dB_{name}"] = rel(mods[name].lora_B.grad, ref[name][3])
