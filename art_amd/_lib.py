@@ -78,6 +78,7 @@ SIGNATURES = {
     "artk_mfma_loop": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
     "artk_mfma_loop16": (_i32, [_p, _i64, _i64, _i32, _p, _p]),
     "artk_stream_copy": (_i32, [_p, _p, _i64, _p]),
+    "artk_gemm_loop_probe": (_i32, [_p, _p, _p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _p, _p]),
     "artk_lds_probe": (_i32, [_i32, _i32, _i32, _p, _i64, _i32, _p, _p]),
 }
 

@@ -4,6 +4,7 @@
 // streaming copy, which gives the matching figure for HBM.
 #include "common.hpp"
 #include "gemm_nt.hpp"
+#include "gemm_4x16.hpp"
 
 namespace artk {
 
@@ -152,6 +153,103 @@ static void launch_lds_probe(int rpd, unsigned blocks, hipStream_t st, const voi
   else lds_probe_kernel<NT, KIND, 3><<<blocks, NT, 0, st>>>(src, iters, cycles);
 }
 
+// Persistent plain GEMM out[n, m] = sum_k Q[n,k] P[m,k] (bf16 out, full tiles only) on a choice of
+// main loop, tile order and ablation switches: what each part of the loop costs on the hardware.
+//   LOOP 0: the library's 8-wave loop (MFMA 32x32x16), 1: its pinned 4-wave loop (32x32x16),
+//        2: the 4-wave loop on MFMA 16x16x32 of gemm_4x16.hpp, with the switches ABL
+// same_tile: every work-group fetches the tiles (b % 8, b % 8) whatever tile it computes, so all
+// fetches hit in L2 (results are then wrong); group: row-operand tiles per column-operand tile of
+// the tile order.  Work-group b reports its core-clock cycles and 100 MHz ticks to cycles[2b..].
+struct LoopProbeParams {
+  const void* P;
+  const void* Q;
+  uint16_t* out;
+  int64_t M, N, K;
+  int MT, NT, group, same_tile;
+  int64_t* cycles;
+};
+
+template <int LOOP, int ABL>
+__global__ __launch_bounds__(LOOP == 0 ? 512 : 256) void loop_probe_kernel(LoopProbeParams p) {
+  constexpr int NI = LOOP == 0 ? 2 : 4;
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  const long long c0 = clock64(), w0 = wall_clock64();
+  const int n_tiles = p.MT * p.NT;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int t = blockIdx.x, mt, nt;
+  tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt, p.group);
+  auto init = [&](TileLoaders<NI>& L, int mt_, int nt_) {
+    const int fm = p.same_tile ? (int)(blockIdx.x & 7) : mt_, fn = p.same_tile ? (int)(blockIdx.x & 7) : nt_;
+    L.init(p.P, p.K, (int64_t)fm * TILE, p.M, p.Q, p.K, (int64_t)fn * TILE, p.N, 0, (int)p.K);
+  };
+  {
+    TileLoaders<NI> first;
+    init(first, mt, nt);
+    first.issue_first(smem);
+  }
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const bool more = t2 < n_tiles;
+    int mt2 = 0, nt2 = 0;
+    if (more) tile_coords(xcd_remap(t2, n_tiles), p.MT, p.NT, mt2, nt2, p.group);
+    TileLoaders<NI> cur;
+    init(cur, mt, nt);
+    if constexpr (LOOP == 2) {
+      TileAcc16 acc;
+      acc.zero();
+      gemm_tile_run_4x16<ABL>(acc, smem, cur);
+      if (more) {
+        TileLoaders<NI> nx;
+        init(nx, mt2, nt2);
+        nx.issue_first(smem);
+      }
+      const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+      for (int nj = 0; nj < 8; ++nj) {
+        const int64_t col = (int64_t)nt * TILE + wn * 128 + nj * 16 + (lane & 15);
+#pragma unroll
+        for (int mi = 0; mi < 8; ++mi) {
+          const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 16 + (lane >> 4) * 4;
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][nj][e];
+          *(bf16x4*)(p.out + col * p.M + m) = o;
+        }
+      }
+    } else {
+      TileAcc<NI> acc;
+      acc.zero();
+      gemm_tile_run(acc, smem, cur);
+      if (more) {
+        TileLoaders<NI> nx;
+        init(nx, mt2, nt2);
+        nx.issue_first(smem);
+      }
+      const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+        const int64_t col = (int64_t)nt * TILE + acc_col<NI>(wn, ni, lane);
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+          store_block_bf16(p.out + col * p.M + (int64_t)mt * TILE + wm * 128 + mi * 32, acc.c[mi][ni], lane >> 5);
+      }
+    }
+    if (!more) break;
+    t = t2;
+    mt = mt2;
+    nt = nt2;
+  }
+  if (threadIdx.x == 0 && p.cycles != nullptr) {
+    p.cycles[2 * blockIdx.x] = clock64() - c0;
+    p.cycles[2 * blockIdx.x + 1] = wall_clock64() - w0;
+  }
+}
+
+template <int ABL>
+static void launch_loop_probe_4x16(const LoopProbeParams& p, unsigned grid, hipStream_t st) {
+  loop_probe_kernel<2, ABL><<<grid, 256, 0, st>>>(p);
+}
+
 __global__ __launch_bounds__(256) void stream_copy_kernel(const uint4* __restrict__ src,
                                                           uint4* __restrict__ dst, int64_t n16) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256)
@@ -206,6 +304,51 @@ int32_t artk_lds_probe(int32_t waves, int32_t kind, int32_t reads_per_dma, const
     if (kind == 0) launch_lds_probe<512, 0>(reads_per_dma, nb, st, src, iters, cycles);
     else if (kind == 1) launch_lds_probe<512, 1>(reads_per_dma, nb, st, src, iters, cycles);
     else launch_lds_probe<512, 2>(reads_per_dma, nb, st, src, iters, cycles);
+  }
+  ARTK_CHECK_LAUNCH();
+  return ARTK_OK;
+}
+
+int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M, int64_t N, int64_t K,
+                             int32_t loop, int32_t ablate, int32_t group, int32_t same_tile, int64_t* cycles,
+                             artk_stream_t stream) {
+  ARTK_CHECK_ARG(P && Q && out, "null pointer argument");
+  ARTK_CHECK_ARG(aligned16(P) && aligned16(Q) && aligned16(out), "pointers must be 16-byte aligned");
+  ARTK_CHECK_ARG(M >= 2048 && N >= 2048 && K >= 128 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0,
+                 "M and N must be multiples of 256 (at least 2048), K a multiple of 64 (at least 128)");
+  ARTK_CHECK_ARG(loop >= 0 && loop <= 2, "loop must be 0 (8-wave), 1 (4-wave 32x32x16) or 2 (4-wave 16x16x32)");
+  ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 && (ablate == 0 || loop == 2),
+                 "ablate: bits 1 (no DMA), 2 (no barrier), 4 (no LDS reads); 6 is not built; only with loop 2");
+  ARTK_CHECK_ARG(group >= 1 && group <= 64, "group must be in 1..64");
+  LoopProbeParams p;
+  p.P = P;
+  p.Q = Q;
+  p.out = (uint16_t*)out;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.MT = (int)(M / TILE);
+  p.NT = (int)(N / TILE);
+  p.group = group;
+  p.same_tile = same_tile != 0;
+  p.cycles = cycles;
+  int cus = 0, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const int64_t tiles = (int64_t)p.MT * p.NT;
+  const unsigned grid = (unsigned)(tiles < cus ? tiles : cus);
+  hipStream_t st = (hipStream_t)stream;
+  if (loop == 0) loop_probe_kernel<0, 0><<<grid, 512, 0, st>>>(p);
+  else if (loop == 1) loop_probe_kernel<1, 0><<<grid, 256, 0, st>>>(p);
+  else switch (ablate) {
+    case 0: launch_loop_probe_4x16<0>(p, grid, st); break;
+    case 1: launch_loop_probe_4x16<1>(p, grid, st); break;
+    case 2: launch_loop_probe_4x16<2>(p, grid, st); break;
+    case 3: launch_loop_probe_4x16<3>(p, grid, st); break;
+    case 4: launch_loop_probe_4x16<4>(p, grid, st); break;
+    case 5: launch_loop_probe_4x16<5>(p, grid, st); break;
+    default: launch_loop_probe_4x16<7>(p, grid, st); break;
   }
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;

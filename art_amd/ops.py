@@ -776,3 +776,26 @@ def lds_probe(waves: int, kind: int, reads_per_dma: int, iters: int, blocks: int
     write_bytes = float(waves) * iters * n_dma * 1024
     return {"read_B_per_clk": read_bytes / core, "dma_write_B_per_clk": write_bytes / core,
             "core_GHz": core / (ticks * 10.0) if ticks > 0 else None}
+
+
+def gemm_loop_probe(p: torch.Tensor, q: torch.Tensor, loop: int = 0, ablate: int = 0, group: int = 8,
+                    same_tile: bool = False, out: Optional[torch.Tensor] = None,
+                    cycles: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out bf16 [N,M] = q [N,K] @ p [M,K]^T on a chosen main loop (0: 8-wave, 1: 4-wave 32x32x16,
+    2: 4-wave 16x16x32), tile-order group and ablation switches (see artk_gemm_loop_probe); the result
+    is only meaningful with ablate == 0 and same_tile False."""
+    M, K = p.shape
+    N = q.shape[0]
+    _need(p, "p", torch.bfloat16)
+    _need(q, "q", torch.bfloat16, (N, K))
+    if out is None:
+        out = torch.empty((N, M), dtype=torch.bfloat16, device=p.device)
+    _need(out, "out", torch.bfloat16, (N, M))
+    if cycles is not None:
+        _need(cycles, "cycles", torch.int64)
+        if cycles.numel() < 2 * torch.cuda.get_device_properties(p.device).multi_processor_count:
+            raise ValueError("cycles needs two int64 per CU")
+    _lib.check(_lib.load().artk_gemm_loop_probe(p.data_ptr(), q.data_ptr(), out.data_ptr(), M, N, K, int(loop),
+                                                int(ablate), int(group), int(bool(same_tile)), _ptr(cycles),
+                                                _stream(p.device)))
+    return out

@@ -1025,6 +1025,36 @@ def bench_ceiling(args, hidden=None, lm_head=None, seconds=0.6):
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
     dst = torch.empty_like(src)
     out["stream_copy"] = run(lambda: ops.stream_copy(src, dst), nbytes=2.0 * src.numel())
+    del src, dst
+    # LDS bytes per clock of a CU, reads alone and with the DMA writes of the GEMM's fill mixed in
+    # (one 1 KiB buffer_load ... lds per 2 or 3 reads: the 4-wave and the 8-wave loop's ratio)
+    lds = {}
+    for name, waves, kind, rpd in (("ds_read_b128_4waves", 4, 1, 0), ("ds_read_b128_8waves", 8, 1, 0),
+                                   ("ds_read_b64_tr_b16_8waves", 8, 2, 0), ("ds_read_b128_4waves_dma", 4, 1, 2),
+                                   ("ds_read_b128_8waves_dma", 8, 1, 3), ("ds_read_b64_tr_b16_8waves_dma", 8, 2, 3)):
+        ops.lds_probe(waves, kind, rpd, 200, blocks, dev)
+        lds[name] = ops.lds_probe(waves, kind, rpd, 20000, blocks, dev)
+    out["lds_bytes_per_clk_per_cu"] = lds
+    if not args.no_secondary:
+        # what each part of the main loop costs: the persistent plain GEMM on the same shape, bf16 output,
+        # on the library's loops and on the 4-wave MFMA 16x16x32 loop with parts switched off
+        probe_out = torch.empty((chunk, V), dtype=torch.bfloat16, device=dev)
+        cyc = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
+        rows = (("8wave_32x32x16_group8", 0, 0, 8, False), ("8wave_32x32x16_group4", 0, 0, 4, False),
+                ("4wave_32x32x16_group4", 1, 0, 4, False), ("4wave_16x16x32_group4", 2, 0, 4, False),
+                ("4wave_16x16x32_group8", 2, 0, 8, False), ("4wave_16x16x32_all_fetches_hit_L2", 2, 0, 4, True),
+                ("4wave_16x16x32_no_wait_no_barrier", 2, 2, 4, False), ("4wave_16x16x32_no_fill", 2, 1, 4, False),
+                ("4wave_16x16x32_no_fill_no_barrier", 2, 3, 4, False),
+                ("4wave_16x16x32_no_lds_reads", 2, 4, 4, False),
+                ("4wave_16x16x32_mfma_and_stores_only", 2, 7, 4, False))
+        table = {}
+        for name, loop, abl, grp, same in rows:
+            rec = run(lambda: ops.gemm_loop_probe(lm_head, h, loop=loop, ablate=abl, group=grp, same_tile=same,
+                                                  out=probe_out, cycles=cyc), flop=gemm_flop)
+            c = cyc.view(-1, 2).double().cpu()
+            rec["core_ghz_in_kernel"] = float((c[:, 0].sum() / (c[:, 1].sum() * 10.0)).item())
+            table[name] = rec
+        out["main_loop_parts"] = table
     return out
 
 

@@ -473,6 +473,20 @@ int32_t artk_mfma_loop(const void* operands, int64_t n_operands, int64_t iters, 
 int32_t artk_mfma_loop16(const void* operands, int64_t n_operands, int64_t iters, int32_t blocks,
                          float* sink, artk_stream_t stream);
 int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_t stream);
+/* artk_gemm_loop_probe: persistent plain NT GEMM out[n,m] = sum_k Q[n,k] P[m,k] (bf16 [N,M]; M, N
+ *   multiples of 256, K of 64) on a choice of main loop and tile order, with switches that take
+ *   parts of the loop away, to measure what each part costs under the part's power limit.
+ *   loop 0: the library's 8-wave loop; 1: its 4-wave loop with pinned instruction order (both MFMA
+ *   32x32x16); 2: a 4-wave loop on MFMA 16x16x32.  ablate (loop 2 only; results are then wrong):
+ *   bit 1 no fill of the LDS stages inside the loop, bit 2 no wait for the fill and no work-group
+ *   barrier, bit 4 no LDS fragment reads.  group: row-operand tiles walked per column-operand tile
+ *   by consecutive tile ids (the library uses 8, or 4 when the row operand streams from HBM).
+ *   same_tile != 0: every work-group fetches the same 8 operand tiles whatever it computes, so every
+ *   fetch hits in L2 (results wrong).  cycles int64 [work-groups][2] or NULL: core-clock cycles and
+ *   100 MHz ticks each work-group ran (one work-group per CU). */
+int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M, int64_t N, int64_t K,
+                             int32_t loop, int32_t ablate, int32_t group, int32_t same_tile, int64_t* cycles,
+                             artk_stream_t stream);
 int32_t artk_lds_probe(int32_t waves, int32_t kind, int32_t reads_per_dma, const void* src, int64_t iters,
                        int32_t blocks, int64_t* cycles, artk_stream_t stream);
 

@@ -80,3 +80,26 @@ def test_lds_probe_reports_a_plausible_rate(artk_lib, gpu, waves, kind, rpd):
     assert (r["dma_write_B_per_clk"] > 0) == (rpd > 0)
     with pytest.raises(ValueError):
         ops.lds_probe(3, 0, 0, 1, 1, gpu)
+
+
+@pytest.mark.parametrize("loop,group", [(0, 8), (1, 4), (2, 8), (2, 4)])
+def test_gemm_loop_probe_computes_the_product(artk_lib, gpu, loop, group):
+    """Without ablation switches every loop variant of the probe is a correct GEMM (fp32 matmul of the
+    bf16 inputs, bf16 rounding of the result); with a switch set it still runs to completion."""
+    print(f"gemm_loop_probe loop={loop} group={group}", flush=True)
+    g = torch.Generator().manual_seed(3 + loop)
+    M, N, K = 2304, 2048, 320
+    p = torch.randn(M, K, generator=g).to(torch.bfloat16).to(gpu)
+    q = torch.randn(N, K, generator=g).to(torch.bfloat16).to(gpu)
+    cyc = torch.zeros(2 * torch.cuda.get_device_properties(gpu).multi_processor_count, dtype=torch.int64, device=gpu)
+    out = ops.gemm_loop_probe(p, q, loop=loop, group=group, cycles=cyc)
+    ref = q.float() @ p.float().t()
+    rel = ((out.float() - ref).norm() / ref.norm()).item()
+    assert rel < 4e-3, rel
+    assert int(cyc[0]) > 0 and int(cyc[1]) > 0
+    if loop == 2:
+        for ablate in (1, 2, 4, 7):
+            ops.gemm_loop_probe(p, q, loop=2, ablate=ablate, group=group, same_tile=True)
+        torch.cuda.synchronize()
+    with pytest.raises(ValueError):
+        ops.gemm_loop_probe(p, q, loop=1, ablate=1)
