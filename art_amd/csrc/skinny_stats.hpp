@@ -384,9 +384,16 @@ __device__ __forceinline__ void stats_reduce_one(const StatsReduceJob& j, int R,
     s *= j.scale;
     if (j.transposed) {
       if (j.n_split > 0) {
-        int k = 0;
-        while (k + 1 < j.n_split && e >= j.e_start[k + 1]) ++k;
-        j.outs[k][(int64_t)(e - j.e_start[k]) * j.n + row] = s;
+        // (constant indices only: a run-time index into the job would send it through scratch memory)
+        float* dst = j.outs[0];
+        int e0 = 0;
+#pragma unroll
+        for (int k = 1; k < 4; ++k)
+          if (k < j.n_split && e >= j.e_start[k]) {
+            dst = j.outs[k];
+            e0 = j.e_start[k];
+          }
+        dst[(int64_t)(e - e0) * j.n + row] = s;
       } else {
         j.out[(int64_t)e * j.n + row] = s;
       }
@@ -398,8 +405,9 @@ __device__ __forceinline__ void stats_reduce_one(const StatsReduceJob& j, int R,
 }
 
 __global__ __launch_bounds__(256) static void stats_reduce_kernel(StatsReduceJob a, StatsReduceJob b, int R, int nblk_a) {
-  const bool first = (int)blockIdx.x < nblk_a;
-  stats_reduce_one(first ? a : b, R, (int64_t)(first ? blockIdx.x : blockIdx.x - nblk_a) * 256 + threadIdx.x);
+  // (each job is used where it lies, among the kernel arguments: a selected copy would live in scratch memory)
+  if ((int)blockIdx.x < nblk_a) stats_reduce_one(a, R, (int64_t)blockIdx.x * 256 + threadIdx.x);
+  else stats_reduce_one(b, R, (int64_t)(blockIdx.x - nblk_a) * 256 + threadIdx.x);
 }
 
 struct StatsGeom {

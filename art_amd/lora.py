@@ -164,8 +164,15 @@ class _FusedLoRAFn(torch.autograd.Function):
                       else g.reshape(-1, g.shape[-1]).to(torch.bfloat16).contiguous())
         dx, dAs, dBs = ops.lora_linear_multi_bwd(g2, x2, [ops.transposed_weight(w) for w in weights], list(A16),
                                                  list(B16), list(xas), scale)
-        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, *([None] * (2 * n)),
-                *[d.to(t) for d, t in zip(dAs, a_dt)], *[d.to(t) for d, t in zip(dBs, b_dt)])
+        # gradients in the parameters' dtypes: one multi-tensor copy instead of a cast per tensor
+        grads, want = list(dAs) + list(dBs), list(a_dt) + list(b_dt)
+        cast = [i for i, (g_, t) in enumerate(zip(grads, want)) if g_.dtype != t]
+        if cast:
+            dst = [torch.empty_like(grads[i], dtype=want[i]) for i in cast]
+            torch._foreach_copy_(dst, [grads[i] for i in cast])
+            for i, d in zip(cast, dst):
+                grads[i] = d
+        return (dx.view(*lead, x2.shape[-1]).to(x_dt), None, None, *([None] * (2 * n)), *grads)
 
 
 class FusedLoRALinear(nn.Module):

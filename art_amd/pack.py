@@ -206,23 +206,31 @@ class RowStager:
     def rows(self, tensors: PackedTensors):
         """Yields the rows of `tensors` (host tensors or the memory maps of
         `packed_tensors_from_dir`) as dicts of device tensors [1, S].  A yielded dict stays
-        valid until the generator is advanced twice more; work on it must be enqueued on the
-        stream that is current when the generator is advanced."""
+        valid until the generator is advanced once more (advancing hands its device buffers to
+        the copy of the row after next); work on it must be enqueued, before that, on the
+        stream that is current when the generator is advanced.  Closing or abandoning the
+        generator early is safe: the slot of the last yielded row is released then."""
         n = tensors["tokens"].shape[0]
         if n == 0:
             return
         self._stage(tensors, 0, self.slots[0])
-        for i in range(n):
-            consumer = torch.cuda.current_stream(self.device)
-            if i >= 1:
-                # everything the consumer enqueued for row i-1 precedes this point of its stream
-                self.slots[(i - 1) % self.DEPTH]["released"].record(consumer)
-            if i + 1 < n:
-                self._stage(tensors, i + 1, self.slots[(i + 1) % self.DEPTH])
-            slot = self.slots[i % self.DEPTH]
-            consumer.wait_event(slot["copied"])
-            yield dict(slot["dev"])
-        self.slots[(n - 1) % self.DEPTH]["released"].record(torch.cuda.current_stream(self.device))
+        pending = None   # slot of the row the consumer holds, not yet released
+        try:
+            for i in range(n):
+                consumer = torch.cuda.current_stream(self.device)
+                if pending is not None:
+                    # everything the consumer enqueued for row i-1 precedes this point of its stream
+                    pending["released"].record(consumer)
+                    pending = None
+                if i + 1 < n:
+                    self._stage(tensors, i + 1, self.slots[(i + 1) % self.DEPTH])
+                slot = self.slots[i % self.DEPTH]
+                consumer.wait_event(slot["copied"])
+                pending = slot
+                yield dict(slot["dev"])
+        finally:
+            if pending is not None:
+                pending["released"].record(torch.cuda.current_stream(self.device))
 
     def to_device(self, tensors: PackedTensors, row: int) -> PackedTensors:
         """One row, ready on the current stream (fresh device tensors, no overlap)."""

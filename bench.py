@@ -28,14 +28,15 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E peak
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None until
 # measured for the workload.  Source: profiles/lmhead_fwd_c3_pmc.md
-TRAFFIC_BYTES = {"c3": 2.05e10, "c1": None}
+TRAFFIC_BYTES = {"c3": 1.58e10, "c1": None}  # 7.34e6 x 2 KiB fetched + 0.70e6 KiB written per forward launch
 # moe_gemm_kernel, mean bytes per launch over the 4 launches of the step with gate|up fused (FETCH_SIZE x 2 KiB +
-# WRITE_SIZE x 1 KiB, the factors a 1 GiB copy gives): 949 MB read + 210 MB written
-MOE_TRAFFIC_BYTES = 1.16e9
-# lora_multi_gemm_kernel on the gate|up forward (8192 x 2048 -> 11008 + 11008): filled in from
-# profiles/lora_c2_pmc.md
-LORA_TRAFFIC_BYTES = None
-LORA_TRAFFIC_SOURCE = None
+# WRITE_SIZE x 1 KiB, the factors a 1 GiB copy gives): 1166 MB read + 211 MB written
+MOE_TRAFFIC_BYTES = 1.38e9
+# lora_multi_gemm_kernel, mean of the two gate|up launches (8192 x 2048 -> 11008 + 11008): y 1.41 GB read + 0.37 GB
+# written, dx 1.08 GB read + 0.03 GB written
+LORA_TRAFFIC_BYTES = 1.45e9
+LORA_TRAFFIC_SOURCE = ("profiles/lora_c2_kernel_trace.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of "
+                       "this command, scaled by a 1 GiB copy; not measured in this run)")
 MOE_TRAFFIC_SOURCE = ("profiles/moe_c5_kernel_trace.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of "
                       "this command, scaled by a 1 GiB copy; not measured in this run)")
 TRAFFIC_SOURCE = {"c3": "profiles/lmhead_fwd_c3_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier "

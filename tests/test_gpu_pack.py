@@ -75,3 +75,11 @@ def test_pack_roundtrip_stager_fused_loss(artk_lib, gpu, tmp_path):
     for i, row in enumerate(stager.rows(loaded)):
         assert torch.equal(row["tokens"].cpu(), packed["tokens"][i:i + 1])
         assert torch.equal(row["assistant_mask"].cpu(), packed["assistant_mask"][i:i + 1])
+    # a pass that is abandoned after its first row releases the slot it held: the next pass is intact
+    it = stager.rows(loaded)
+    first = next(it)
+    assert torch.equal(first["tokens"].cpu(), packed["tokens"][0:1])
+    it.close()
+    for i, row in enumerate(stager.rows(loaded)):
+        assert torch.equal(row["tokens"].cpu(), packed["tokens"][i:i + 1])
+        assert torch.equal(row["advantages"].cpu(), packed["advantages"][i:i + 1])
