@@ -1042,6 +1042,7 @@ def bench_ceiling(args, hidden=None, lm_head=None, seconds=0.6):
         probe_out = torch.empty((chunk, V), dtype=torch.bfloat16, device=dev)
         cyc = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
         rows = (("8wave_32x32x16_group8", 0, 0, 8, False), ("8wave_32x32x16_group4", 0, 0, 4, False),
+                ("8wave_32x32x16_group2", 0, 0, 2, False), ("8wave_32x32x16_group16", 0, 0, 16, False),
                 ("4wave_32x32x16_group4", 1, 0, 4, False), ("4wave_16x16x32_group4", 2, 0, 4, False),
                 ("4wave_16x16x32_group8", 2, 0, 8, False), ("4wave_16x16x32_all_fetches_hit_L2", 2, 0, 4, True),
                 ("4wave_16x16x32_no_wait_no_barrier", 2, 2, 4, False), ("4wave_16x16x32_no_fill", 2, 1, 4, False),
