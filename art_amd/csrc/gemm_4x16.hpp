@@ -159,4 +159,111 @@ __device__ __forceinline__ void gemm_tile_run_4x16(TileAcc16& acc, char* smem, c
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the MFMAs above are invisible to the compiler
 }
 
+// ----------------------------------------------------------------------------
+// The 8-wave work-group shape (2 x 4 waves, wave tile 128 x 64, two waves per SIMD) on MFMA
+// 16x16x32: 8 x 4 tiles of 16 x 16 per wave, 128 accumulators per lane.  A K = 32 step is 32 MFMAs,
+// 12 fragment reads of the next step and 4 DMA instructions; the compiler orders them under
+// scheduling-group barriers as in the 8-wave loop of gemm_nt.hpp (the second wave of the SIMD
+// covers what stalls remain).
+struct TileAcc16x8 {
+  floatx4 c[8][4];  // [mi][nj]: row wm*128 + mi*16 + (lane/16)*4 + e, column wn*64 + nj*16 + lane%16
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[i][j][e] = 0.f;
+  }
+};
+struct Frags16x8 {
+  bf16x8 p[8], q[4];
+};
+__device__ __forceinline__ void load_frags16x8(Frags16x8& f, const char* sp, const char* sq, int off) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) f.q[j] = *(const bf16x8*)(sq + off + j * 2048);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f.p[i] = *(const bf16x8*)(sp + off + i * 2048);
+}
+__device__ __forceinline__ void mma_frags16x8(TileAcc16x8& acc, const Frags16x8& f) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.p[i], f.q[j], acc.c[i][j], 0, 0, 0);
+}
+
+__device__ __forceinline__ void gemm_tile_run_8x16(TileAcc16x8& acc, char* smem, const TileLoaders<2>& L) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int wm = wave >> 2, wn = wave & 3;
+  const OperandLoader<2>& lp = L.lp;
+  const OperandLoader<2>& lq = L.lq;
+  const int k_begin = L.k_begin, k_end = L.k_end;
+  int off[2];
+  {
+    const int rl = lane & 15;
+    const int f = swz(rl);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) off[ks] = rl * 128 + (((ks * 4 + (lane >> 4)) ^ f) << 4);
+  }
+  const int p_wave_off = wm * 128 * 128;
+  const int q_wave_off = OPER_STAGE_BYTES + wn * 64 * 128;
+  const int nk = (k_end - k_begin) / BK;
+
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (nk > 1) {
+    lp.template issue<0, 2, 50>(smem + STAGE_BYTES, wave, k_begin + BK);
+    lq.template issue<0, 2, 50>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
+  }
+  Frags16x8 fa, fb;
+  load_frags16x8(fa, smem + p_wave_off, smem + q_wave_off, off[0]);
+
+  auto k_step = [&](int kt, auto late_tag, auto ahead_tag) {
+    constexpr bool LATE = decltype(late_tag)::value, AHEAD = decltype(ahead_tag)::value;
+    char* cur = smem + (kt & 1) * STAGE_BYTES;
+    char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
+    if constexpr (LATE) {
+      const int k1 = k_begin + (kt + 1) * BK;
+      lp.template issue<2, 4, 51>(nxt, wave, k1);
+      lq.template issue<2, 4, 51>(nxt + OPER_STAGE_BYTES, wave, k1);
+    }
+    load_frags16x8(fb, cur + p_wave_off, cur + q_wave_off, off[1]);
+    mma_frags16x8(acc, fa);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      if (LATE && i < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    if constexpr (AHEAD) {
+      const int k2 = k_begin + (kt + 2) * BK;
+      lp.template issue<0, 2, 52>(cur, wave, k2);
+      lq.template issue<0, 2, 52>(cur + OPER_STAGE_BYTES, wave, k2);
+    }
+    // (after the last K-step this reads the idle stage: values nobody uses)
+    load_frags16x8(fa, nxt + p_wave_off, nxt + q_wave_off, off[0]);
+    mma_frags16x8(acc, fb);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      if (AHEAD && i < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+  for (int kt = 0; kt < nk - 2; ++kt) k_step(kt, yes{}, yes{});
+  if (nk > 1) k_step(nk - 2, yes{}, no{});
+  k_step(nk - 1, no{}, no{});
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+}
+
 }  // namespace artk

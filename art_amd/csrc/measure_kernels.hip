@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "gemm_nt.hpp"
 #include "gemm_4x16.hpp"
+#include "gemm_half.hpp"
 
 namespace artk {
 
@@ -156,7 +157,9 @@ static void launch_lds_probe(int rpd, unsigned blocks, hipStream_t st, const voi
 // Persistent plain GEMM out[n, m] = sum_k Q[n,k] P[m,k] (bf16 out, full tiles only) on a choice of
 // main loop, tile order and ablation switches: what each part of the loop costs on the hardware.
 //   LOOP 0: the library's 8-wave loop (MFMA 32x32x16), 1: its pinned 4-wave loop (32x32x16),
-//        2: the 4-wave loop on MFMA 16x16x32 of gemm_4x16.hpp, with the switches ABL
+//        2: the 4-wave loop on MFMA 16x16x32 of gemm_4x16.hpp, with the switches ABL,
+//        3: the 8-wave shape on MFMA 16x16x32 (gemm_4x16.hpp), 4: 256 x 128 tiles, two work-groups per CU
+//           (gemm_half.hpp)
 // same_tile: every work-group fetches the tiles (b % 8, b % 8) whatever tile it computes, so all
 // fetches hit in L2 (results are then wrong); group: row-operand tiles per column-operand tile of
 // the tile order.  Work-group b reports its core-clock cycles and 100 MHz ticks to cycles[2b..].
@@ -170,12 +173,63 @@ struct LoopProbeParams {
 };
 
 template <int LOOP, int ABL>
-__global__ __launch_bounds__(LOOP == 0 ? 512 : 256) void loop_probe_kernel(LoopProbeParams p) {
-  constexpr int NI = LOOP == 0 ? 2 : 4;
-  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+__global__ __launch_bounds__(LOOP == 0 || LOOP == 3 ? 512 : 256, LOOP == 4 ? 2 : 1) void loop_probe_kernel(
+    LoopProbeParams p) {
+  constexpr int NI = LOOP == 0 || LOOP == 3 ? 2 : 4;
+  __shared__ __attribute__((aligned(1024))) char smem[LOOP == 4 ? HALF_LDS_BYTES : GEMM_LDS_BYTES];
   const long long c0 = clock64(), w0 = wall_clock64();
-  const int n_tiles = p.MT * p.NT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if constexpr (LOOP == 4) {
+    // 256 x 128 tiles, two work-groups per CU
+    const int NT2 = p.NT * 2, n_tiles2 = p.MT * NT2;
+    int t = blockIdx.x, mt, nt;
+    tile_coords(xcd_remap(t, n_tiles2), p.MT, NT2, mt, nt, p.group);
+    auto init = [&](HalfLoaders& L, int mt_, int nt_) {
+      const int fm = p.same_tile ? (int)(blockIdx.x & 7) : mt_, fn = p.same_tile ? (int)(blockIdx.x & 7) : nt_;
+      L.init(p.P, p.K, (int64_t)fm * TILE, p.M, p.Q, p.K, (int64_t)fn * HALF_Q, p.N, 0, (int)p.K);
+    };
+    {
+      HalfLoaders first;
+      init(first, mt, nt);
+      first.issue_first(smem);
+    }
+    for (;;) {
+      const int t2 = t + gridDim.x;
+      const bool more = t2 < n_tiles2;
+      int mt2 = 0, nt2 = 0;
+      if (more) tile_coords(xcd_remap(t2, n_tiles2), p.MT, NT2, mt2, nt2, p.group);
+      TileAcc<2> acc;
+      acc.zero();
+      {
+        HalfLoaders cur;
+        init(cur, mt, nt);
+        gemm_half_run(acc, smem, cur);
+      }
+      if (more) {
+        HalfLoaders nx;
+        init(nx, mt2, nt2);
+        nx.issue_first(smem);
+      }
+      const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const int64_t col = (int64_t)nt * HALF_Q + wn * 64 + ni * 32 + (lane & 31);
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+          store_block_bf16(p.out + col * p.M + (int64_t)mt * TILE + wm * 128 + mi * 32, acc.c[mi][ni], lane >> 5);
+      }
+      if (!more) break;
+      t = t2;
+      mt = mt2;
+      nt = nt2;
+    }
+    if (threadIdx.x == 0 && p.cycles != nullptr && blockIdx.x < gridDim.x / 2) {
+      p.cycles[2 * blockIdx.x] = clock64() - c0;
+      p.cycles[2 * blockIdx.x + 1] = wall_clock64() - w0;
+    }
+    return;
+  }
+  const int n_tiles = p.MT * p.NT;
   int t = blockIdx.x, mt, nt;
   tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt, p.group);
   auto init = [&](TileLoaders<NI>& L, int mt_, int nt_) {
@@ -216,7 +270,29 @@ __global__ __launch_bounds__(LOOP == 0 ? 512 : 256) void loop_probe_kernel(LoopP
           *(bf16x4*)(p.out + col * p.M + m) = o;
         }
       }
-    } else {
+    } else if constexpr (LOOP == 3) {
+      TileAcc16x8 acc;
+      acc.zero();
+      gemm_tile_run_8x16(acc, smem, cur);
+      if (more) {
+        TileLoaders<NI> nx;
+        init(nx, mt2, nt2);
+        nx.issue_first(smem);
+      }
+      const int wm = wave >> 2, wn = wave & 3;
+#pragma unroll
+      for (int nj = 0; nj < 4; ++nj) {
+        const int64_t col = (int64_t)nt * TILE + wn * 64 + nj * 16 + (lane & 15);
+#pragma unroll
+        for (int mi = 0; mi < 8; ++mi) {
+          const int64_t m = (int64_t)mt * TILE + wm * 128 + mi * 16 + (lane >> 4) * 4;
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc.c[mi][nj][e];
+          *(bf16x4*)(p.out + col * p.M + m) = o;
+        }
+      }
+    } else if constexpr (LOOP != 4) {
       TileAcc<NI> acc;
       acc.zero();
       gemm_tile_run(acc, smem, cur);
@@ -316,7 +392,9 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
   ARTK_CHECK_ARG(aligned16(P) && aligned16(Q) && aligned16(out), "pointers must be 16-byte aligned");
   ARTK_CHECK_ARG(M >= 2048 && N >= 2048 && K >= 128 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0,
                  "M and N must be multiples of 256 (at least 2048), K a multiple of 64 (at least 128)");
-  ARTK_CHECK_ARG(loop >= 0 && loop <= 2, "loop must be 0 (8-wave), 1 (4-wave 32x32x16) or 2 (4-wave 16x16x32)");
+  ARTK_CHECK_ARG(loop >= 0 && loop <= 4,
+                 "loop must be 0 (8-wave), 1 (4-wave 32x32x16), 2 (4-wave 16x16x32), 3 (8-wave 16x16x32) or 4 "
+                 "(256 x 128 tiles, two work-groups per CU)");
   ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 && (ablate == 0 || loop == 2),
                  "ablate: bits 1 (no DMA), 2 (no barrier), 4 (no LDS reads); 6 is not built; only with loop 2");
   ARTK_CHECK_ARG(group >= 1 && group <= 64, "group must be in 1..64");
@@ -341,6 +419,11 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
   hipStream_t st = (hipStream_t)stream;
   if (loop == 0) loop_probe_kernel<0, 0><<<grid, 512, 0, st>>>(p);
   else if (loop == 1) loop_probe_kernel<1, 0><<<grid, 256, 0, st>>>(p);
+  else if (loop == 3) loop_probe_kernel<3, 0><<<grid, 512, 0, st>>>(p);
+  else if (loop == 4) {
+    const int64_t tiles2 = tiles * 2;
+    loop_probe_kernel<4, 0><<<(unsigned)(tiles2 < 2 * cus ? tiles2 : 2 * cus), 256, 0, st>>>(p);
+  }
   else switch (ablate) {
     case 0: launch_loop_probe_4x16<0>(p, grid, st); break;
     case 1: launch_loop_probe_4x16<1>(p, grid, st); break;

@@ -1038,13 +1038,16 @@ def bench_ceiling(args, hidden=None, lm_head=None, seconds=0.6):
     out["lds_bytes_per_clk_per_cu"] = lds
     if not args.no_secondary:
         # what each part of the main loop costs: the persistent plain GEMM on the same shape, bf16 output,
-        # on the library's loops and on the 4-wave MFMA 16x16x32 loop with parts switched off
+        # on the library's loops, on the MFMA 16x16x32 loops (4-wave with parts switched off, 8-wave) and on
+        # 256 x 128 tiles with two work-groups per CU
         probe_out = torch.empty((chunk, V), dtype=torch.bfloat16, device=dev)
         cyc = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
         rows = (("8wave_32x32x16_group8", 0, 0, 8, False), ("8wave_32x32x16_group4", 0, 0, 4, False),
                 ("8wave_32x32x16_group2", 0, 0, 2, False), ("8wave_32x32x16_group16", 0, 0, 16, False),
                 ("4wave_32x32x16_group4", 1, 0, 4, False), ("4wave_16x16x32_group4", 2, 0, 4, False),
-                ("4wave_16x16x32_group8", 2, 0, 8, False), ("4wave_16x16x32_all_fetches_hit_L2", 2, 0, 4, True),
+                ("4wave_16x16x32_group8", 2, 0, 8, False), ("8wave_16x16x32_group4", 3, 0, 4, False),
+                ("two_workgroups_per_cu_256x128_group4", 4, 0, 4, False),
+                ("4wave_16x16x32_all_fetches_hit_L2", 2, 0, 4, True),
                 ("4wave_16x16x32_no_wait_no_barrier", 2, 2, 4, False), ("4wave_16x16x32_no_fill", 2, 1, 4, False),
                 ("4wave_16x16x32_no_fill_no_barrier", 2, 3, 4, False),
                 ("4wave_16x16x32_no_lds_reads", 2, 4, 4, False),

@@ -82,7 +82,7 @@ def test_lds_probe_reports_a_plausible_rate(artk_lib, gpu, waves, kind, rpd):
         ops.lds_probe(3, 0, 0, 1, 1, gpu)
 
 
-@pytest.mark.parametrize("loop,group", [(0, 8), (1, 4), (2, 8), (2, 4)])
+@pytest.mark.parametrize("loop,group", [(0, 8), (1, 4), (2, 8), (2, 4), (3, 4), (4, 8), (4, 4)])
 def test_gemm_loop_probe_computes_the_product(artk_lib, gpu, loop, group):
     """Without ablation switches every loop variant of the probe is a correct GEMM (fp32 matmul of the
     bf16 inputs, bf16 rounding of the result); with a switch set it still runs to completion."""
