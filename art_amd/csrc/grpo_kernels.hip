@@ -82,16 +82,67 @@ struct FwdParams {
   int VT, TT;
 };
 
-// Per-position (max, sum-exp) over this wave's 128 vocabulary rows and the gather
-// of the target logit.  RAGGED: the tile reaches past the last vocabulary row and
-// those rows are left out (last tile only).
-template <bool RAGGED>
-__device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt, int wm,
-                                             int64_t vbase, const int64_t (&y)[FWD_NI],
-                                             const int (&col)[FWD_NI], int n) {
+// Epilogue of one logits tile, per wave: its 128 vocabulary rows x 64 positions.
+//
+// For every position: the (reference, sum-exp) partial over the wave's vocabulary rows and the
+// gather of the target logit.  The reference of the partial is the maximum of the 128 logits,
+// except for a position whose row goes to the stash: there it is the row's own reference
+// ref[row], so that one exponential per logit, exp(z - ref), serves both the sum and the
+// stash (the exponentials are the epilogue's cost: they run at a quarter of the vector rate
+// while the matrix pipe idles).  Partials of one position merge whatever their references are.
+// If a logit exceeds its row's reference by more than fp32's exponent range the sum is
+// infinite; such a position's partial is recomputed against the maximum (its stash row holds
+// infinities and the backward drops the row, see splitk_reduce_kernel).
+//
+// STASH: bf16 exp(z - ref) of the positions in `need`.  A lane holds 4 consecutive vocabulary
+// rows of one position, so stored straight from the registers a row would go out in 8-byte
+// pieces, 32 positions per store instruction: the L2 then takes one 16-byte request per piece
+// pair and the wave waits for thousands of them.  Instead the wave transposes 32 positions at
+// a time through `scratch` (EPI_LDS_PER_WAVE bytes of LDS per wave that nothing else uses during
+// the epilogue: 32 rows of 256 bytes at a pitch of 272, which keeps the 8-byte writes and the
+// 16-byte reads free of bank conflicts), and 16 lanes store 256 contiguous bytes of a position.
+// RAGGED: the tile reaches past the last vocabulary row and those rows are left out.
+constexpr int EPI_PITCH = 272;
+constexpr int EPI_LDS_PER_WAVE = 32 * EPI_PITCH;                                  // 8704
+constexpr int EPI_LDS_EXTRA = 8 * EPI_LDS_PER_WAVE - STAGE_BYTES;                 // beyond the idle GEMM stage
+struct EpiRow {  // what the epilogue needs to know about one position of the tile
+  int64_t y;     // target id, -1 past the end
+  int col;
+  bool want;
+  float ref;
+};
+// Issued before the next tile's first DMA stage, so that waiting for these values does not wait
+// for that stage (loads complete in order).
+template <bool STASH>
+__device__ __forceinline__ void lmhead_epilogue_rows(const FwdParams& p, int tt, int n, EpiRow (&row)[FWD_NI]) {
   const int lane = threadIdx.x & 63;
+  const int wn = wave_n<FWD_NI>(threadIdx.x >> 6);
+#pragma unroll
+  for (int ni = 0; ni < FWD_NI; ++ni) {
+    EpiRow& r = row[ni];
+    r.col = tt * TILE + acc_col<FWD_NI>(wn, ni, lane);
+    r.y = r.col < n ? target_id(p.ids, p.rows.token(r.col), p.S, p.shift) : (int64_t)-1;
+    r.want = STASH && r.col < n && (p.need == nullptr || p.need[r.col] != 0);
+    r.ref = r.want ? p.ref[r.col] : 0.f;
+  }
+}
+
+template <bool STASH, bool RAGGED>
+__device__ __forceinline__ void lmhead_fwd_epilogue_impl(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt,
+                                                         int tt, int n, const EpiRow (&row)[FWD_NI],
+                                                         char* scratch) {
+  static_assert(FWD_NI == 2, "the LDS transpose is laid out for 8 waves of 128 x 64");
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave_m<FWD_NI>(wave), wn = wave_n<FWD_NI>(wave);
   const int half = lane >> 5;
-  const int vleft = (int)(p.V - vbase < 128 ? p.V - vbase : 128);  // valid rows of this wave
+  const int c = lane & 31;
+  const int64_t vbase = (int64_t)vt * TILE + wm * 128;  // first vocab row of this wave
+  const int vleft = (int)(p.V - vbase < 128 ? p.V - vbase : 128);  // valid rows of this wave (may be <= 0)
+  char* my = scratch + wave * EPI_LDS_PER_WAVE;
+  char* my_w = my + c * EPI_PITCH + half * 8;                              // this lane's 8-byte pieces
+  const char* my_r = my + (lane >> 4) * EPI_PITCH + (lane & 15) * 16;      // 16 bytes of row i*4 + lane/16
+
 #pragma unroll
   for (int ni = 0; ni < FWD_NI; ++ni) {
     // A position's 128 logits of this wave: 64 in this lane, 64 in lane^32.
@@ -105,22 +156,54 @@ __device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const F
         m = fmaxf(m, (RAGGED && r >= vleft) ? -INFINITY : z);
       }
     m = fmaxf(m, __shfl_xor(m, 32, 64));
-    const float mb = (m == -INFINITY ? 0.f : m) * LOG2E;
+    float mr = row[ni].want ? row[ni].ref : m;  // reference of this position's partial
+    const float mb = (mr == -INFINITY ? 0.f : mr) * LOG2E;
     float l = 0.f;
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][j], LOG2E, -mb));
-        l += (RAGGED && r >= vleft) ? 0.f : e;
+      for (int q = 0; q < 4; ++q) {
+        float e[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int r = mi * 32 + q * 8 + half * 4 + k;
+          e[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][q * 4 + k], LOG2E, -mb));
+          if (RAGGED && r >= vleft) e[k] = 0.f;
+          l += e[k];
+        }
+        if (STASH) {
+          bf16x4 o;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o[k] = (__bf16)e[k];
+          *(bf16x4*)(my_w + (mi * 8 + q * 2) * 8) = o;  // rows mi*32 + q*8 + half*4 .. +3 of position c
+        }
       }
     l += __shfl_xor(l, 32, 64);
-    if (lane < 32 && col[ni] < n)
-      p.part[(int64_t)(vt * 2 + wm) * p.Tc + col[ni]] = make_float2(m, l);
+    if (STASH) {
+      const bool ovf = row[ni].want && !(l <= 3.0e38f);
+      if (__any(ovf)) {
+        const float mb2 = (m == -INFINITY ? 0.f : m) * LOG2E;
+        float l2 = 0.f;
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][j], LOG2E, -mb2));
+            l2 += (RAGGED && r >= vleft) ? 0.f : e;
+          }
+        l2 += __shfl_xor(l2, 32, 64);
+        if (ovf) {
+          mr = m;
+          l = l2;
+        }
+      }
+    }
+    if (lane < 32 && row[ni].col < n)
+      p.part[(int64_t)(vt * 2 + wm) * p.Tc + row[ni].col] = make_float2(mr, l);
 
     // Gather: exactly one lane of one wave of the whole grid holds logit[y].
-    const int64_t rel = y[ni] - vbase;
+    const int64_t rel = row[ni].y - vbase;
     const bool hit = rel >= 0 && rel < 128 && ((((int)rel) >> 2) & 1) == half;
     if (__any(hit)) {
       float s = 0.f;
@@ -131,62 +214,42 @@ __device__ __forceinline__ void lse_epilogue(const TileAcc<FWD_NI>& acc, const F
           const int r = mi * 32 + (j >> 2) * 8 + half * 4 + (j & 3);
           s = (r == (int)rel) ? acc.c[mi][ni][j] : s;
         }
-      if (hit) p.sel[col[ni]] = s;
+      if (hit) p.sel[row[ni].col] = s;
+    }
+
+    if (STASH) {
+      const uint32_t mask = (uint32_t)__ballot(row[ni].want);  // bit i: position i of these 32 (both halves agree)
+      if (mask != 0) {
+        __builtin_amdgcn_wave_barrier();
+        const int k16 = lane & 15;
+        const int64_t v0 = vbase + k16 * 8;
+        const int64_t col0 = (int64_t)tt * TILE + wn * 64 + ni * 32;
+        uint16_t* dst = p.stash + (col0 + (lane >> 4)) * p.V + v0;
+        const uint32_t mine = v0 < p.V ? mask >> (lane >> 4) : 0u;  // bit 4i: position i*4 + lane/16
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          uint4 d[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) d[i] = *(const uint4*)(my_r + (h * 4 + i) * 4 * EPI_PITCH);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if ((mine >> (4 * (h * 4 + i))) & 1u) *(uint4*)(dst + (int64_t)(h * 4 + i) * 4 * p.V) = d[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
     }
   }
 }
 
-// Epilogue of one logits tile: optional bf16 stash of the rows the backward needs,
-// then the (max, sumexp) partials and the target gather.
 template <bool STASH>
 __device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, const FwdParams& p, int vt,
-                                                    int tt, int n) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wm = wave_m<FWD_NI>(wave), wn = wave_n<FWD_NI>(wave);
-  const int half = lane >> 5;
-  const int64_t vbase = (int64_t)vt * TILE + wm * 128;  // first vocab row of this wave
-
-  // Targets of this lane's positions (issued early: consumed after the reductions).
-  int64_t y[FWD_NI];
-  int col[FWD_NI];
-#pragma unroll
-  for (int ni = 0; ni < FWD_NI; ++ni) {
-    col[ni] = tt * TILE + acc_col<FWD_NI>(wn, ni, lane);
-    y[ni] = col[ni] < n ? target_id(p.ids, p.rows.token(col[ni]), p.S, p.shift) : (int64_t)-1;
-  }
-
-  if (STASH) {
-#pragma unroll
-    for (int ni = 0; ni < FWD_NI; ++ni) {
-      const bool want = col[ni] < n && (p.need == nullptr || p.need[col[ni]] != 0);
-      if (!__any(want)) continue;
-      if (want) {
-        uint16_t* row = p.stash + (int64_t)col[ni] * p.V;
-        const float nref = -p.ref[col[ni]] * LOG2E;
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            int64_t v = vbase + mi * 32 + q * 8 + half * 4;
-            if (v < p.V) {
-              bf16x4 o;
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                o[e] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(acc.c[mi][ni][q * 4 + e], LOG2E, nref));
-              *(bf16x4*)(row + v) = o;
-            }
-          }
-      }
-    }
-  }
-
-  // The accumulators are only read from here on (writing to them would make the
-  // compiler shuttle all of them between the accumulation and the vector registers).
+                                                    int tt, int n, const EpiRow (&row)[FWD_NI], char* scratch) {
+  // The accumulators are only read (writing to them would make the compiler shuttle all of
+  // them between the accumulation and the vector registers).
   if ((int64_t)vt * TILE + TILE > p.V)
-    lse_epilogue<true>(acc, p, vt, wm, vbase, y, col, n);
+    lmhead_fwd_epilogue_impl<STASH, true>(acc, p, vt, tt, n, row, scratch);
   else
-    lse_epilogue<false>(acc, p, vt, wm, vbase, y, col, n);
+    lmhead_fwd_epilogue_impl<STASH, false>(acc, p, vt, tt, n, row, scratch);
 }
 
 // Next tile of this work-group at or after id `t` (stride = grid size) whose
@@ -206,7 +269,7 @@ __device__ __forceinline__ bool lmhead_next_tile(const FwdParams& p, int n_tiles
 // prologue latency of a tile hides behind the epilogue of the previous one.
 template <bool STASH>
 __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
-  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
+  __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES + (STASH ? EPI_LDS_EXTRA : 0)];
   const int n_tiles = p.VT * p.TT;
   const int n = p.rows.n();
   int t = blockIdx.x, vt, tt;
@@ -228,6 +291,8 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
                p.rows.row_token);
       gemm_tile_run(acc, smem, cur);
     }
+    EpiRow row[FWD_NI];
+    lmhead_epilogue_rows<STASH>(p, tt, n, row);
     if (more) {
       // loaders are rebuilt rather than kept: alive through the epilogue they cost registers
       TileLoaders<FWD_NI> nxt;
@@ -235,7 +300,9 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
                p.rows.row_token);
       nxt.issue_first(smem);
     }
-    lmhead_fwd_epilogue<STASH>(acc, p, vt, tt, n);
+    // the second LDS stage (and what lies behind it) is idle until the next tile's first barrier:
+    // scratch of the epilogue
+    lmhead_fwd_epilogue<STASH>(acc, p, vt, tt, n, row, smem + STAGE_BYTES);
     if (!more) break;
     t = t2;
     vt = vt2;

@@ -172,7 +172,9 @@ def test_fused_target_far_under_the_maximum_is_dropped_and_counted(artk_lib, gpu
 
 def test_fused_no_grad_runs_the_forward_half_only(artk_lib, gpu):
     """Under torch.no_grad() (an evaluation pass) the loss comes from the forward kernels alone
-    and equals the training pass's loss and logprobs bit for bit."""
+    and equals the training pass's loss and logprobs up to fp32 rounding (the training pass sums a
+    stashed row's exponentials against the row's target logit, the evaluation pass against the
+    running maximum)."""
     T, H, V = 512, 128, 4096
     case = synthetic.make_grpo_case("t", 98, T, H, V, 4, 4, 0.5)
     oracle_case(case, 256)   # fills in the old logprobs
@@ -189,9 +191,13 @@ def test_fused_no_grad_runs_the_forward_half_only(artk_lib, gpu):
     _, n_fwd = ops.profile_collect(ops.PROF_LMHEAD_FWD)
     ops.profile_enable(False)
     assert n_fwd >= 1 and n_bwd == 0
-    assert loss2.item() == loss.item()
-    assert torch.equal(logprob2, logprob)
-    assert metrics2["policy_loss"].item() == metrics["policy_loss"].item()
+    # (the loss is a mean of signed terms of order 1e-2 that nearly cancel)
+    assert abs(loss2.item() - loss.item()) <= 1e-4 * abs(loss.item()) + 1e-7
+    assert torch.equal(torch.isnan(logprob2), torch.isnan(logprob))
+    ok = ~torch.isnan(logprob)
+    assert (logprob2[ok] - logprob[ok]).abs().max().item() <= 1e-5
+    assert abs(metrics2["policy_loss"].item() - metrics["policy_loss"].item()) <= (
+        1e-4 * abs(metrics["policy_loss"].item()) + 1e-7)
     assert metrics2["dropped_rows"].item() == 0.0
     assert not loss2.requires_grad
 
@@ -380,7 +386,7 @@ def test_full_size_windows_and_properties(artk_lib, gpu, name):
     args, s, lp, dh, new = run_full_size(case, gpu, 4096)
     count = grpo_oracle.shift_tensor(case.assistant_mask, False).sum().item()
     assert s[3].item() == count                       # integer mask count, bit-exact
-    assert torch.equal(lp, new)                        # fused forward == forward-only kernel
+    assert same_logprobs(lp, new)                      # fused forward == forward-only kernel
     # windows: start of the row, a trajectory boundary, the end of the row
     L = T // (32 if name == "c3" else 16)
     for start in (0, 3 * L - 40, T - 96):
@@ -426,6 +432,16 @@ def test_full_size_windows_and_properties(artk_lib, gpu, name):
     assert dh4[dead.to(gpu)].abs().max().item() == 0.0
 
 
+def same_logprobs(a, b, tol=2e-5):
+    """The fused step and the forward-only entry point agree up to fp32 rounding: the fused step sums
+    a stashed row's exponentials against the row's target logit, the forward-only kernel against the
+    running maximum.  NaN (no target) in the same places."""
+    if not torch.equal(torch.isnan(a), torch.isnan(b)):
+        return False
+    ok = ~torch.isnan(a)
+    return (a[ok] - b[ok]).abs().max().item() <= tol
+
+
 def chunk_bounds(T, V):
     """First positions of the chunks the library forms by itself (chunk_tokens = 0): about 6000
     positions per chunk, the batch's 256-position tiles spread evenly over the chunks."""
@@ -456,7 +472,7 @@ def test_full_size_library_chunking_and_independent_loss(artk_lib, gpu, name):
     args, s, lp, dh, new = run_full_size(case, gpu, 0)
     count = grpo_oracle.shift_tensor(case.assistant_mask, False).sum().item()
     assert s[3].item() == count
-    assert torch.equal(lp, new)
+    assert same_logprobs(lp, new)
     bounds = chunk_bounds(T, V)
     assert len(bounds) >= 3 and bounds[1] - bounds[0] != bounds[-1] - bounds[-2]  # uneven chunks
     starts = (bounds[1] - 48, bounds[-1] - 48, bounds[-1] + 700, T - 96)
