@@ -189,6 +189,15 @@ __device__ __forceinline__ void store_block_bf16(uint16_t* dst, const floatx16& 
   }
 }
 
+// LDS scratch of an epilogue that transposes a wave's 128 x 64 block (8-wave shape) 32 columns
+// at a time: 32 rows of 256 bytes at a pitch of 272 per wave (8-byte writes down a column and
+// 16-byte reads along a row are then free of bank conflicts).  Eight of them cover the second
+// GEMM stage, which is idle during an epilogue (the next tile's first DMA stage only fills the
+// first), plus EPI_LDS_EXTRA bytes behind it.
+constexpr int EPI_PITCH = 272;
+constexpr int EPI_LDS_PER_WAVE = 32 * EPI_PITCH;                   // 8704
+constexpr int EPI_LDS_EXTRA = 8 * EPI_LDS_PER_WAVE - STAGE_BYTES;  // 4096
+
 // The two operand loaders and the K range of one tile.  Separate from the main
 // loop so that a kernel that walks several tiles can set up the next tile's
 // loaders and start its first DMA stage before the current tile's epilogue

@@ -102,9 +102,6 @@ struct FwdParams {
 // the epilogue: 32 rows of 256 bytes at a pitch of 272, which keeps the 8-byte writes and the
 // 16-byte reads free of bank conflicts), and 16 lanes store 256 contiguous bytes of a position.
 // RAGGED: the tile reaches past the last vocabulary row and those rows are left out.
-constexpr int EPI_PITCH = 272;
-constexpr int EPI_LDS_PER_WAVE = 32 * EPI_PITCH;                                  // 8704
-constexpr int EPI_LDS_EXTRA = 8 * EPI_LDS_PER_WAVE - STAGE_BYTES;                 // beyond the idle GEMM stage
 struct EpiRow {  // what the epilogue needs to know about one position of the tile
   int64_t y;     // target id, -1 past the end
   int col;
