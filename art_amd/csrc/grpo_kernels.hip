@@ -249,16 +249,26 @@ __device__ __forceinline__ void lmhead_fwd_epilogue(const TileAcc<FWD_NI>& acc, 
     lmhead_fwd_epilogue_impl<STASH, false>(acc, p, vt, tt, n, row, scratch);
 }
 
-// Next tile of this work-group at or after id `t` (stride = grid size) whose
-// token tile is not past the last row; false when there is none.
-__device__ __forceinline__ bool lmhead_next_tile(const FwdParams& p, int n_tiles, int n, int& t, int& vt,
-                                                 int& tt) {
-  for (; t < n_tiles; t += gridDim.x) {
-    tile_coords(xcd_remap(t, n_tiles), p.VT, p.TT, vt, tt, TILE_GROUP_STREAMING);
-    if (tt * TILE < n) return true;
+// The order of the tiles of one launch: TT position tiles that hold rows (in compact mode their
+// number is known only on the device) and how many vocabulary tiles an XCD's 32 work-groups walk
+// per position tile.  With plenty of position tiles a patch is 4 x 8 (gemm_nt.hpp); with fewer
+// than a patch is wide it takes more vocabulary tiles instead, so that the 32 still work on one
+// patch (measured at 2048 x 896 x 151936: 8 position tiles 0.897 -> 0.876 ms per step with 8
+// instead of 4, the 4 position tiles of its compact rows 0.861 -> 0.644 ms; at 3584 and 21-22
+// position tiles 4 stays best, 20.4 against 20.8 ms).
+struct FwdOrder {
+  int TT, n_tiles, group;
+  __device__ __forceinline__ FwdOrder(const FwdParams& p, int n) {
+    const int live = (n + TILE - 1) / TILE;
+    TT = live < p.TT ? live : p.TT;
+    n_tiles = p.VT * TT;
+    group = TT >= 12 ? TILE_GROUP_STREAMING : (TT >= 4 ? 8 : (TT >= 2 ? 16 : 32));
   }
-  return false;
-}
+  // Tile id t (< n_tiles) -> vocabulary tile, position tile.
+  __device__ __forceinline__ void coords(const FwdParams& p, int t, int& vt, int& tt) const {
+    tile_coords(xcd_remap(t, n_tiles), p.VT, TT, vt, tt, group);
+  }
+};
 
 // Persistent work-groups (one per CU): each walks tiles t, t + grid, ...  The
 // next tile's loaders are set up before the current tile's main loop and its
@@ -267,10 +277,11 @@ __device__ __forceinline__ bool lmhead_next_tile(const FwdParams& p, int n_tiles
 template <bool STASH>
 __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES + (STASH ? EPI_LDS_EXTRA : 0)];
-  const int n_tiles = p.VT * p.TT;
   const int n = p.rows.n();
+  const FwdOrder order(p, n);
   int t = blockIdx.x, vt, tt;
-  if (!lmhead_next_tile(p, n_tiles, n, t, vt, tt)) return;
+  if (t >= order.n_tiles) return;
+  order.coords(p, t, vt, tt);
   {
     TileLoaders<FWD_NI> first;
     first.init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H,
@@ -278,8 +289,10 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
     first.issue_first(smem);
   }
   for (;;) {
-    int t2 = t + gridDim.x, vt2 = 0, tt2 = 0;
-    const bool more = lmhead_next_tile(p, n_tiles, n, t2, vt2, tt2);
+    const int t2 = t + gridDim.x;
+    int vt2 = 0, tt2 = 0;
+    const bool more = t2 < order.n_tiles;
+    if (more) order.coords(p, t2, vt2, tt2);
     TileAcc<FWD_NI> acc;
     acc.zero();
     {
