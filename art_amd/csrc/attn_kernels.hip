@@ -28,6 +28,7 @@ namespace artk {
 constexpr int ATT_BM = 256;    // queries per work-group
 constexpr int ATT_BN = 64;     // keys per tile
 constexpr int ATT_STAGES = 3;
+constexpr float ATT_LAZY = 8.f;   // forward: how far a score may exceed the exponentials' reference (log2 units)
 constexpr int ATT_MAX_KB = 1024;  // key blocks per row the list in LDS can hold
 constexpr int ATT_BQ2 = 64;    // dK/dV kernel: queries per tile
 constexpr int ATT_BK2 = 128;   // dK/dV kernel: keys per work-group (4 key groups x 32)
@@ -436,12 +437,9 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
       }
     }
 
-    // scale, mask, running max
+    // mask, running max (of the raw scores: the scale is positive and rides in the exponent's
+    // multiply-add below)
     float mloc = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) sc[kt][j] *= p.scale_log2e;
     if (partial) {
       const int* codes = (const int*)(st + G::CODE_OFF);
 #pragma unroll
@@ -461,27 +459,34 @@ __global__ __launch_bounds__(512) void attn_fwd_kernel(AttnFwdParams p) {
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int j = 0; j < 16; ++j) mloc = fmaxf(mloc, sc[kt][j]);
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-    const float m_new = fmaxf(m_run, mloc);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64)) * p.scale_log2e;
+    // The reference of the exponentials follows the running maximum lazily: it moves only when
+    // some query of the wave has a score more than ATT_LAZY (in units of log2) above it, so the
+    // 64 output accumulators are rescaled on few tiles instead of on most early ones.  Until
+    // then exponentials are at most 2^ATT_LAZY, which fp32 sums and bf16 operands hold without
+    // loss; the final division by the sum is the same.
+    const bool move = __any(mloc > m_run + ATT_LAZY);
     float lsum = 0.f;
     bf16x8 pf[4];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float e = __builtin_amdgcn_exp2f(sc[kt][j] - m_new);
-        lsum += e;
-        pf[2 * kt + j / 8][j % 8] = (__bf16)e;
-      }
-    l_run = l_run * alpha + lsum;
-    if (__any(alpha != 1.f)) {
+    if (move) {
+      const float m_new = fmaxf(m_run, mloc);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
         for (int j = 0; j < 16; ++j) o[dt][j] *= alpha;
     }
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][j], p.scale_log2e, -m_run));
+        lsum += e;
+        pf[2 * kt + j / 8][j % 8] = (__bf16)e;
+      }
+    l_run += lsum;
 
     // O^T += V^T P^T, V^T fragments by transposing reads of the V tile
     const char* vt = st + G::V_OFF;
@@ -1069,6 +1074,7 @@ int32_t artk_attn_fwd(const void* q, const void* k, const void* v, const void* p
                               v_stride_s, v_stride_h, o_stride_s, o_stride_h};
   int32_t rc = attn_check(S, Hq, Hkv, D, strides, 8);
   if (rc) return rc;
+  ARTK_CHECK_ARG(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
   (void)workspace; (void)workspace_bytes;
   AttnPlan pl;
   attn_plan_layout(const_cast<void*>(plan), (size_t)1 << 40, S, pl);

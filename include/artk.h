@@ -270,7 +270,7 @@ int32_t artk_transpose_bf16_batched(const void* in, void* out, int64_t n, int64_
  *   multiples of 8), likewise k, v ([S, Hkv, D]) and out; query head h reads
  *   key/value head h / (Hq / Hkv).  lse is f32 [Hq, S].
  * artk_attn_bwd: dq, dk, dv (bf16, same addressing as q, k, v) from d_out.
- * Requires S % 256 == 0, S <= 65536, D in {64, 128}.
+ * Requires S % 256 == 0, S <= 65536, D in {64, 128}, scale > 0 (forward).
  * ------------------------------------------------------------------------- */
 size_t artk_attn_plan_bytes(int64_t S);
 int32_t artk_attn_plan(const int64_t* group_ids, const int64_t* parent_ids, int64_t S, void* plan,
