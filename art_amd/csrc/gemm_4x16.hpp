@@ -193,6 +193,7 @@ __device__ __forceinline__ void mma_frags16x8(TileAcc16x8& acc, const Frags16x8&
       acc.c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.p[i], f.q[j], acc.c[i][j], 0, 0, 0);
 }
 
+template <int ABL = 0>
 __device__ __forceinline__ void gemm_tile_run_8x16(TileAcc16x8& acc, char* smem, const TileLoaders<2>& L) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -214,23 +215,25 @@ __device__ __forceinline__ void gemm_tile_run_8x16(TileAcc16x8& acc, char* smem,
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  if (nk > 1) {
-    lp.template issue<0, 2, 50>(smem + STAGE_BYTES, wave, k_begin + BK);
-    lq.template issue<0, 2, 50>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
+  if (nk > 1 && !(ABL & ABL_NO_DMA)) {
+    lp.template issue<0, 2, 500 + ABL>(smem + STAGE_BYTES, wave, k_begin + BK);
+    lq.template issue<0, 2, 500 + ABL>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
   }
   Frags16x8 fa, fb;
   load_frags16x8(fa, smem + p_wave_off, smem + q_wave_off, off[0]);
+  if constexpr ((ABL & ABL_NO_LDS_READ) != 0) fb = fa;
 
   auto k_step = [&](int kt, auto late_tag, auto ahead_tag) {
     constexpr bool LATE = decltype(late_tag)::value, AHEAD = decltype(ahead_tag)::value;
     char* cur = smem + (kt & 1) * STAGE_BYTES;
     char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
-    if constexpr (LATE) {
+    constexpr bool DMA = !(ABL & ABL_NO_DMA), RD = !(ABL & ABL_NO_LDS_READ);
+    if constexpr (LATE && DMA) {
       const int k1 = k_begin + (kt + 1) * BK;
-      lp.template issue<2, 4, 51>(nxt, wave, k1);
-      lq.template issue<2, 4, 51>(nxt + OPER_STAGE_BYTES, wave, k1);
+      lp.template issue<2, 4, 510 + ABL>(nxt, wave, k1);
+      lq.template issue<2, 4, 510 + ABL>(nxt + OPER_STAGE_BYTES, wave, k1);
     }
-    load_frags16x8(fb, cur + p_wave_off, cur + q_wave_off, off[1]);
+    if constexpr (RD) load_frags16x8(fb, cur + p_wave_off, cur + q_wave_off, off[1]);
     mma_frags16x8(acc, fa);
 #pragma unroll
     for (int i = 0; i < 12; ++i) {
@@ -239,15 +242,17 @@ __device__ __forceinline__ void gemm_tile_run_8x16(TileAcc16x8& acc, char* smem,
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
-    if constexpr (AHEAD) {
+    if constexpr (!(ABL & ABL_NO_BARRIER)) {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+    if constexpr (AHEAD && DMA) {
       const int k2 = k_begin + (kt + 2) * BK;
-      lp.template issue<0, 2, 52>(cur, wave, k2);
-      lq.template issue<0, 2, 52>(cur + OPER_STAGE_BYTES, wave, k2);
+      lp.template issue<0, 2, 520 + ABL>(cur, wave, k2);
+      lq.template issue<0, 2, 520 + ABL>(cur + OPER_STAGE_BYTES, wave, k2);
     }
     // (after the last K-step this reads the idle stage: values nobody uses)
-    load_frags16x8(fa, nxt + p_wave_off, nxt + q_wave_off, off[0]);
+    if constexpr (RD) load_frags16x8(fa, nxt + p_wave_off, nxt + q_wave_off, off[0]);
     mma_frags16x8(acc, fb);
 #pragma unroll
     for (int i = 0; i < 12; ++i) {

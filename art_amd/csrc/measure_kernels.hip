@@ -273,7 +273,7 @@ __global__ __launch_bounds__(LOOP == 0 || LOOP == 3 ? 512 : 256, LOOP == 4 ? 2 :
     } else if constexpr (LOOP == 3) {
       TileAcc16x8 acc;
       acc.zero();
-      gemm_tile_run_8x16(acc, smem, cur);
+      gemm_tile_run_8x16<ABL>(acc, smem, cur);
       if (more) {
         TileLoaders<NI> nx;
         init(nx, mt2, nt2);
@@ -395,8 +395,9 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
   ARTK_CHECK_ARG(loop >= 0 && loop <= 4,
                  "loop must be 0 (8-wave), 1 (4-wave 32x32x16), 2 (4-wave 16x16x32), 3 (8-wave 16x16x32) or 4 "
                  "(256 x 128 tiles, two work-groups per CU)");
-  ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 && (ablate == 0 || loop == 2),
-                 "ablate: bits 1 (no DMA), 2 (no barrier), 4 (no LDS reads); 6 is not built; only with loop 2");
+  ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 && (ablate == 0 || loop == 2 || (loop == 3 && ablate != 3)),
+                 "ablate: bits 1 (no DMA), 2 (no barrier), 4 (no LDS reads); 6 is not built (nor 3 with loop 3); only "
+                 "with loops 2 and 3");
   ARTK_CHECK_ARG(group >= 1 && group <= 64, "group must be in 1..64");
   LoopProbeParams p;
   p.P = P;
@@ -419,7 +420,16 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
   hipStream_t st = (hipStream_t)stream;
   if (loop == 0) loop_probe_kernel<0, 0><<<grid, 512, 0, st>>>(p);
   else if (loop == 1) loop_probe_kernel<1, 0><<<grid, 256, 0, st>>>(p);
-  else if (loop == 3) loop_probe_kernel<3, 0><<<grid, 512, 0, st>>>(p);
+  else if (loop == 3) {
+    switch (ablate) {
+      case 0: loop_probe_kernel<3, 0><<<grid, 512, 0, st>>>(p); break;
+      case 1: loop_probe_kernel<3, 1><<<grid, 512, 0, st>>>(p); break;
+      case 2: loop_probe_kernel<3, 2><<<grid, 512, 0, st>>>(p); break;
+      case 4: loop_probe_kernel<3, 4><<<grid, 512, 0, st>>>(p); break;
+      case 5: loop_probe_kernel<3, 5><<<grid, 512, 0, st>>>(p); break;
+      default: loop_probe_kernel<3, 7><<<grid, 512, 0, st>>>(p); break;
+    }
+  }
   else if (loop == 4) {
     const int64_t tiles2 = tiles * 2;
     loop_probe_kernel<4, 0><<<(unsigned)(tiles2 < 2 * cus ? tiles2 : 2 * cus), 256, 0, st>>>(p);

@@ -479,7 +479,8 @@ int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_
  *   loop 0: the library's 8-wave loop; 1: its 4-wave loop with pinned instruction order (both MFMA
  *   32x32x16); 2: a 4-wave loop on MFMA 16x16x32; 3: the 8-wave shape on MFMA 16x16x32; 4: 256 x 128
  *   tiles on 4 waves with a 3-stage ring of K = 32 stages, two work-groups per CU (cycles then holds
- *   the first work-group of each pair).  ablate (loop 2 only; results are then wrong):
+ *   the first work-group of each pair).  ablate (loops 2 and 3; results are then wrong; 6, and 3 with loop 3, are
+ *   not built):
  *   bit 1 no fill of the LDS stages inside the loop, bit 2 no wait for the fill and no work-group
  *   barrier, bit 4 no LDS fragment reads.  group: row-operand tiles walked per column-operand tile
  *   by consecutive tile ids (the library uses 8, or 4 when the row operand streams from HBM).

@@ -97,9 +97,9 @@ def test_gemm_loop_probe_computes_the_product(artk_lib, gpu, loop, group):
     rel = ((out.float() - ref).norm() / ref.norm()).item()
     assert rel < 4e-3, rel
     assert int(cyc[0]) > 0 and int(cyc[1]) > 0
-    if loop == 2:
+    if loop in (2, 3):
         for ablate in (1, 2, 4, 7):
-            ops.gemm_loop_probe(p, q, loop=2, ablate=ablate, group=group, same_tile=True)
+            ops.gemm_loop_probe(p, q, loop=loop, ablate=ablate, group=group, same_tile=True)
         torch.cuda.synchronize()
     with pytest.raises(ValueError):
         ops.gemm_loop_probe(p, q, loop=1, ablate=1)
