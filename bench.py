@@ -630,6 +630,32 @@ def bench_attn(args):
                        "unit": "TFLOP/s", "frac": kv["frac"], "traffic": None, "launch_ms": kv["launch_ms"]}
     res["plan_ms"] = timed(lambda: ops.attn_plan(group.to(dev), parent.to(dev)), 3, 1) * 1e3
     if not args.no_secondary:
+        # The same kernels on a dense causal row of the same shape (one group: every tile full but
+        # the diagonal), where the per-kernel rate is not blurred by partly visible tiles.
+        zero = torch.zeros(S, dtype=torch.int64, device=dev)
+        dplan = ops.attn_plan(zero, zero)
+        n_dense = S * (S + 1) // 2
+
+        def dense_step():
+            o, l = ops.attn_fwd(q, k, v, dplan)
+            return ops.attn_bwd(q, k, v, o, l, d_out, dplan)
+
+        dense_step()
+        torch.cuda.synchronize()
+        ops.profile_enable(True)
+        for _ in range(3):
+            dense_step()
+        torch.cuda.synchronize()
+        dprof = {name: ops.profile_collect(kind) for name, kind in
+                 (("attn_fwd_kernel", ops.PROF_ATTN_FWD), ("attn_bwd_kv_kernel", ops.PROF_ATTN_BWD_KV),
+                  ("attn_bwd_dq_kernel", ops.PROF_ATTN_BWD_Q))}
+        ops.profile_enable(False)
+        dunit = 2.0 * n_dense * D * Hq
+        res["dense_causal_row"] = {
+            name: {"launch_ms": ms / max(n, 1),
+                   "tflops_executed": executed[name] * dunit / (ms / max(n, 1) * 1e-3) / 1e12}
+            for name, (ms, n) in dprof.items()}
+        del dplan
         # The reference's method on the same GPU: the dense [1, S, S] bias of calculate_attn_bias
         # (src/art/local/train.py:177-215) handed to torch's scaled_dot_product_attention.
         import torch.nn.functional as F
