@@ -220,8 +220,8 @@ struct TileLoaders {
   // reading stage 0 (true at kernel start and after gemm_tile_run returns).
   __device__ __forceinline__ void issue_first(char* smem) const {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    lp.template issue<0, 2 * NI>(smem, wave, k_begin);
-    lq.template issue<0, 2 * NI>(smem + OPER_STAGE_BYTES, wave, k_begin);
+    lp.template issue<0, 2 * NI, 77>(smem, wave, k_begin);
+    lq.template issue<0, 2 * NI, 77>(smem + OPER_STAGE_BYTES, wave, k_begin);
   }
 };
 
@@ -242,7 +242,7 @@ struct TileLoaders {
 // that would reach past the end of the K range.
 __device__ __forceinline__ void gemm_tile_run_pinned(TileAcc<4>& acc, char* smem, const TileLoaders<4>& L);
 
-template <int NI, int NQ = NI>
+template <int NI, int NQ = NI, bool ALL_EARLY = false>
 __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const TileLoaders<NI>& L) {
   if constexpr (NI == 4) {
     gemm_tile_run_pinned(acc, smem, L);  // one wave per SIMD: the order is pinned (see below)
@@ -270,12 +270,17 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
   const int nk = (k_end - k_begin) / BK;
 
-  constexpr int EARLY = NI;  // DMA instructions per operand issued right after the barrier
+  // DMA instructions per operand issued right after the barrier that frees their buffer, the rest at the
+  // start of the next K-step.  All of them early (a full K-step of lead) pays where most row-operand
+  // panels miss in L2 (grouped GEMMs whose weights serve two or three tiles: +1-2 %); elsewhere the split
+  // is faster (lm_head forward at a hidden size of 896: 6 %, LoRA linear: 1.4 %).
+  constexpr int EARLY = ALL_EARLY ? DI : NI;
+  constexpr int TG = NQ + (ALL_EARLY ? 10 : 0);  // issue<> tag
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (nk > 1) {
-    lp.template issue<0, EARLY, NQ>(smem + STAGE_BYTES, wave, k_begin + BK);
-    lq.template issue<0, EARLY, NQ>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
+    lp.template issue<0, EARLY, TG>(smem + STAGE_BYTES, wave, k_begin + BK);
+    lq.template issue<0, EARLY, TG>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
   }
   Frags<NI> f0, f1;
   load_frags<NI, NQ>(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
@@ -293,8 +298,8 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (LATE) {
       const int k1 = k_begin + (kt + 1) * BK;
-      lp.template issue<EARLY, DI, NQ>(nxt, wave, k1);
-      lq.template issue<EARLY, DI, NQ>(nxt + OPER_STAGE_BYTES, wave, k1);
+      lp.template issue<EARLY, DI, TG>(nxt, wave, k1);
+      lq.template issue<EARLY, DI, TG>(nxt + OPER_STAGE_BYTES, wave, k1);
     }
     load_frags<NI, NQ>(f1, sp, sq, off[1]);
     mma_frags<NI, NQ>(acc, f0);
@@ -336,8 +341,8 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (AHEAD) {
       const int k2 = k_begin + (kt + 2) * BK;
-      lp.template issue<0, EARLY, NQ>(cur, wave, k2);
-      lq.template issue<0, EARLY, NQ>(cur + OPER_STAGE_BYTES, wave, k2);
+      lp.template issue<0, EARLY, TG>(cur, wave, k2);
+      lq.template issue<0, EARLY, TG>(cur + OPER_STAGE_BYTES, wave, k2);
     }
     // (after the last K-step this reads the idle stage: values nobody uses)
     load_frags<NI, NQ>(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
@@ -355,6 +360,7 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
       for (int i = 0; i < 6; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (AHEAD && i < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (AHEAD && i + 6 < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
@@ -372,14 +378,15 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
 // gemm_tile_run for a tile whose column operand has only `ncols` (<= 256) rows that anybody
 // stores: a wave computes only those of its NI 32-column tiles that contain such a column
-// (wave-uniform choice; every variant executes the same barriers).  8-wave shape only.
+// (wave-uniform choice; every variant executes the same barriers).  8-wave shape only.  Its caller
+// is the grouped GEMM, so the whole fill of a stage is requested right after the barrier.
 __device__ __forceinline__ void gemm_tile_run_cols(TileAcc<2>& acc, char* smem, const TileLoaders<2>& L,
                                                    int ncols) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int left = ncols - wave_n<2>(wave) * 64;  // columns of this wave that are stored
-  if (left > 32) gemm_tile_run<2, 2>(acc, smem, L);
-  else if (left > 0) gemm_tile_run<2, 1>(acc, smem, L);
-  else gemm_tile_run<2, 0>(acc, smem, L);
+  if (left > 32) gemm_tile_run<2, 2, true>(acc, smem, L);
+  else if (left > 0) gemm_tile_run<2, 1, true>(acc, smem, L);
+  else gemm_tile_run<2, 0, true>(acc, smem, L);
 }
 
 // ----------------------------------------------------------------------------
