@@ -216,12 +216,21 @@ struct TileLoaders {
     k_begin = kb;
     k_end = ke;
   }
+  // DMA instructions LO .. HI-1 of this wave's share of both operands, K offset k0, into the stage at
+  // `stage`.  (TAG is unused: callers that are themselves instantiated several times pass a distinct
+  // value each.)
+  template <int LO, int HI, int TAG>
+  __device__ __forceinline__ void issue(char* stage, int wave, int k0) const {
+    lp.template issue<LO, HI, TAG>(stage, wave, k0);
+    lq.template issue<LO, HI, TAG>(stage + OPER_STAGE_BYTES, wave, k0);
+  }
+  // DMA instructions that issue<LO, LO + 1> stands for (the instruction order is pinned with it).
+  static constexpr int DMA_PER_INDEX = 2;
   // First K stage into LDS stage 0.  No wave of the work-group may still be
   // reading stage 0 (true at kernel start and after gemm_tile_run returns).
   __device__ __forceinline__ void issue_first(char* smem) const {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    lp.template issue<0, 2 * NI, 77>(smem, wave, k_begin);
-    lq.template issue<0, 2 * NI, 77>(smem + OPER_STAGE_BYTES, wave, k_begin);
+    issue<0, 2 * NI, 77>(smem, wave, k_begin);
   }
 };
 
@@ -241,20 +250,38 @@ struct TileLoaders {
 // The loop body has no branches; the last two K-steps are peeled off without the DMA
 // that would reach past the end of the K range.
 __device__ __forceinline__ void gemm_tile_run_pinned(TileAcc<4>& acc, char* smem, const TileLoaders<4>& L);
+template <int NQ, bool ALL_EARLY, class LOADERS>
+__device__ __forceinline__ void gemm_tile_run_8(TileAcc<2>& acc, char* smem, const LOADERS& L,
+                                                std::integral_constant<int, NQ>,
+                                                std::integral_constant<bool, ALL_EARLY>);
 
-template <int NI, int NQ = NI, bool ALL_EARLY = false>
-__device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const TileLoaders<NI>& L) {
+// Instruction-order group: one MFMA, then N DMA issues, then one LDS read.
+template <int N>
+__device__ __forceinline__ void mfma_dma_read_group() {
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(0x020, N, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+}
+
+template <int NI, int NQ = NI, bool ALL_EARLY = false, class LOADERS = TileLoaders<NI>>
+__device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, const LOADERS& L) {
   if constexpr (NI == 4) {
     gemm_tile_run_pinned(acc, smem, L);  // one wave per SIMD: the order is pinned (see below)
     return;
+  } else {
+    gemm_tile_run_8(acc, smem, L, std::integral_constant<int, NQ>{}, std::integral_constant<bool, ALL_EARLY>{});
   }
+}
+template <int NQ, bool ALL_EARLY, class LOADERS>
+__device__ __forceinline__ void gemm_tile_run_8(TileAcc<2>& acc, char* smem, const LOADERS& L,
+                                                std::integral_constant<int, NQ>,
+                                                std::integral_constant<bool, ALL_EARLY>) {
+  constexpr int NI = 2;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
   constexpr int DI = 2 * NI;
-  const OperandLoader<NI>& lp = L.lp;
-  const OperandLoader<NI>& lq = L.lq;
   const int k_begin = L.k_begin, k_end = L.k_end;
 
   // Per-lane LDS read offsets (within an operand stage) for the 4 K=16 steps.
@@ -279,8 +306,7 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (nk > 1) {
-    lp.template issue<0, EARLY, TG>(smem + STAGE_BYTES, wave, k_begin + BK);
-    lq.template issue<0, EARLY, TG>(smem + STAGE_BYTES + OPER_STAGE_BYTES, wave, k_begin + BK);
+    L.template issue<0, EARLY, TG>(smem + STAGE_BYTES, wave, k_begin + BK);
   }
   Frags<NI> f0, f1;
   load_frags<NI, NQ>(f0, smem + p_wave_off, smem + q_wave_off, off[0]);
@@ -298,8 +324,7 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (LATE) {
       const int k1 = k_begin + (kt + 1) * BK;
-      lp.template issue<EARLY, DI, TG>(nxt, wave, k1);
-      lq.template issue<EARLY, DI, TG>(nxt + OPER_STAGE_BYTES, wave, k1);
+      L.template issue<EARLY, DI, TG + 100>(nxt, wave, k1);
     }
     load_frags<NI, NQ>(f1, sp, sq, off[1]);
     mma_frags<NI, NQ>(acc, f0);
@@ -307,8 +332,8 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
     mma_frags<NI, NQ>(acc, f1);
     load_frags<NI, NQ>(f1, sp, sq, off[3]);
     mma_frags<NI, NQ>(acc, f0);
-    // Interleave: 3 steps of 4*NI MFMAs, 3*(4+NI) LDS reads, 2*(DI-EARLY) DMA issues.
-    constexpr int NLATE = LATE ? 2 * (DI - EARLY) : 0;
+    // Interleave: 3 steps of 4*NI MFMAs, 3*(4+NI) LDS reads, NLATE DMA issues.
+    constexpr int NLATE = LATE ? LOADERS::DMA_PER_INDEX * (DI - EARLY) : 0;
     if constexpr (NI == 4) {
 #pragma unroll
       for (int i = 0; i < NLATE; ++i) {
@@ -341,13 +366,12 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
 
     if constexpr (AHEAD) {
       const int k2 = k_begin + (kt + 2) * BK;
-      lp.template issue<0, EARLY, TG>(cur, wave, k2);
-      lq.template issue<0, EARLY, TG>(cur + OPER_STAGE_BYTES, wave, k2);
+      L.template issue<0, EARLY, TG + 200>(cur, wave, k2);
     }
     // (after the last K-step this reads the idle stage: values nobody uses)
     load_frags<NI, NQ>(f0, nxt + p_wave_off, nxt + q_wave_off, off[0]);
     mma_frags<NI, NQ>(acc, f1);
-    // 4*NI MFMA, 4+NI LDS reads, 2*EARLY DMA issues
+    // 4*NI MFMA, 4+NI LDS reads, NA DMA issues
     if constexpr (NI == 4) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -356,13 +380,13 @@ __device__ __forceinline__ void gemm_tile_run(TileAcc<NI>& acc, char* smem, cons
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     } else {
-#pragma unroll
-      for (int i = 0; i < 6; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (AHEAD && i < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        if (AHEAD && i + 6 < 2 * EARLY) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
+      constexpr int NA = AHEAD ? LOADERS::DMA_PER_INDEX * EARLY : 0;  // spread over the six groups
+      mfma_dma_read_group<NA / 6 + (0 < NA % 6)>();
+      mfma_dma_read_group<NA / 6 + (1 < NA % 6)>();
+      mfma_dma_read_group<NA / 6 + (2 < NA % 6)>();
+      mfma_dma_read_group<NA / 6 + (3 < NA % 6)>();
+      mfma_dma_read_group<NA / 6 + (4 < NA % 6)>();
+      mfma_dma_read_group<NA / 6 + (5 < NA % 6)>();
       __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
     }
   };

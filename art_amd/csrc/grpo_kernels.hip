@@ -8,6 +8,7 @@
 //   src/art/local/train.py:111-151  ratio / clip / KL / weight*mask / normalise
 #include "common.hpp"
 #include "gemm_nt.hpp"
+#include "gemm_plain8.hpp"
 
 #include <math.h>
 
@@ -274,7 +275,29 @@ struct FwdOrder {
 // next tile's loaders are set up before the current tile's main loop and its
 // first DMA stage is started before the current tile's epilogue, so the
 // prologue latency of a tile hides behind the epilogue of the previous one.
-template <bool STASH>
+// Loaders and main loop of one forward tile.  GATHER: the rows of the chunk are compact (row_token
+// maps them to positions and the hidden states are gathered); otherwise both operands are plain
+// panels and the first wave of each SIMD issues all DMA (gemm_plain8.hpp).
+template <bool GATHER>
+struct FwdLoaders : PlainTileLoaders {
+  __device__ __forceinline__ void init_tile(const FwdParams& p, int vt, int tt, int n) {
+    init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H);
+  }
+  __device__ __forceinline__ void run(TileAcc<FWD_NI>& acc, char* smem) const {
+    gemm_tile_run_plain8<false>(acc, smem, *this);
+  }
+};
+template <>
+struct FwdLoaders<true> : TileLoaders<FWD_NI> {
+  __device__ __forceinline__ void init_tile(const FwdParams& p, int vt, int tt, int n) {
+    init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H, p.rows.row_token);
+  }
+  __device__ __forceinline__ void run(TileAcc<FWD_NI>& acc, char* smem) const {
+    gemm_tile_run<FWD_NI, FWD_NI, false>(acc, smem, static_cast<const TileLoaders<FWD_NI>&>(*this));
+  }
+};
+
+template <bool STASH, bool GATHER>
 __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES + (STASH ? EPI_LDS_EXTRA : 0)];
   const int n = p.rows.n();
@@ -283,9 +306,8 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
   if (t >= order.n_tiles) return;
   order.coords(p, t, vt, tt);
   {
-    TileLoaders<FWD_NI> first;
-    first.init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H,
-               p.rows.row_token);
+    FwdLoaders<GATHER> first;
+    first.init_tile(p, vt, tt, n);
     first.issue_first(smem);
   }
   for (;;) {
@@ -296,18 +318,16 @@ __global__ __launch_bounds__(nthreads<FWD_NI>()) void lmhead_fwd_kernel(FwdParam
     TileAcc<FWD_NI> acc;
     acc.zero();
     {
-      TileLoaders<FWD_NI> cur;  // its first stage is already on the way
-      cur.init(p.W, p.H, (int64_t)vt * TILE, p.V, p.hidden, p.H, (int64_t)tt * TILE, n, 0, (int)p.H,
-               p.rows.row_token);
-      gemm_tile_run(acc, smem, cur);
+      FwdLoaders<GATHER> cur;  // its first stage is already on the way
+      cur.init_tile(p, vt, tt, n);
+      cur.run(acc, smem);
     }
     EpiRow row[FWD_NI];
     lmhead_epilogue_rows<STASH>(p, tt, n, row);
     if (more) {
       // loaders are rebuilt rather than kept: alive through the epilogue they cost registers
-      TileLoaders<FWD_NI> nxt;
-      nxt.init(p.W, p.H, (int64_t)vt2 * TILE, p.V, p.hidden, p.H, (int64_t)tt2 * TILE, n, 0, (int)p.H,
-               p.rows.row_token);
+      FwdLoaders<GATHER> nxt;
+      nxt.init_tile(p, vt2, tt2, n);
       nxt.issue_first(smem);
     }
     // the second LDS stage (and what lies behind it) is idle until the next tile's first barrier:
@@ -968,10 +988,15 @@ static int32_t launch_fwd_chunk(const void* hidden, const void* lm_head, const i
   const int n_tiles = p.VT * p.TT;
   const unsigned grid = (unsigned)(n_tiles < num_cus() ? n_tiles : num_cus());
   prof_begin(PROF_LMHEAD_FWD, st);
-  if (stash)
-    lmhead_fwd_kernel<true><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
+  const bool gather = rows.row_token != nullptr;
+  if (stash && gather)
+    lmhead_fwd_kernel<true, true><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
+  else if (stash)
+    lmhead_fwd_kernel<true, false><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
+  else if (gather)
+    lmhead_fwd_kernel<false, true><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
   else
-    lmhead_fwd_kernel<false><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
+    lmhead_fwd_kernel<false, false><<<grid, nthreads<FWD_NI>(), 0, st>>>(p);
   prof_end(PROF_LMHEAD_FWD, st);
   ARTK_CHECK_LAUNCH();
   lse_finalize_kernel<<<(unsigned)((Tc + 15) / 16), 256, 0, st>>>(part, 2 * p.VT, Tc, rows, sel, logprob,

@@ -16,6 +16,7 @@
 // and dA from one pass over x (lora_stats_kernel, skinny_stats.hpp).
 #include "common.hpp"
 #include "gemm_nt.hpp"
+#include "gemm_plain8.hpp"
 #include "lora_common.hpp"
 #include "skinny_stats.hpp"
 
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemm
   int mt, nt;
   tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt);
   {
-    TileLoaders<LORA_NI> first;
+    PlainTileLoaders first;
     first.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
     first.issue_first(smem);
   }
@@ -138,12 +139,12 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_gemm_kernel(LoraGemm
     TileAcc<LORA_NI> acc;
     acc.zero();
     {
-      TileLoaders<LORA_NI> cur;  // its first stage is already on the way
+      PlainTileLoaders cur;  // its first stage is already on the way
       cur.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
-      gemm_tile_run(acc, smem, cur);
+      gemm_tile_run_plain8<false>(acc, smem, cur);
     }
     if (more) {
-      TileLoaders<LORA_NI> nxt;
+      PlainTileLoaders nxt;
       nxt.init(p.P, p.K, (int64_t)mt2 * TILE, p.M, p.Q, p.K, (int64_t)nt2 * TILE, p.N, 0, (int)p.K);
       nxt.issue_first(smem);
     }
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_multi_gemm_kernel(Lo
   lora_multi_locate(p, t, j, mt, nt);
   {
     const LoraSeg& sg = p.seg[p.job[j].seg0];
-    TileLoaders<LORA_NI> first;
+    PlainTileLoaders first;
     first.init(sg.P, sg.K, (int64_t)mt * TILE, p.job[j].M, sg.Q, sg.K, (int64_t)nt * TILE, p.N, 0, (int)sg.K);
     first.issue_first(smem);
   }
@@ -214,16 +215,24 @@ __global__ __launch_bounds__(nthreads<LORA_NI>()) void lora_multi_gemm_kernel(Lo
     const int seg0 = p.job[j].seg0, nseg = p.job[j].nseg;
     TileAcc<LORA_NI> acc;
     acc.zero();
-    for (int s = 0; s < nseg; ++s) {
-      const LoraSeg& sg = p.seg[seg0 + s];
-      TileLoaders<LORA_NI> cur;  // the first segment's first stage is already on the way
-      cur.init(sg.P, sg.K, (int64_t)mt * TILE, M, sg.Q, sg.K, (int64_t)nt * TILE, p.N, 0, (int)sg.K);
-      if (s > 0) cur.issue_first(smem);
-      gemm_tile_run(acc, smem, cur);
+    // (one branch around all segments, not one per segment: see gemm_plain8.hpp)
+    if (plain8_leader()) {
+      for (int s = 0; s < nseg; ++s) {
+        const LoraSeg& sg = p.seg[seg0 + s];
+        PlainTileLoaders cur;  // the first segment's first stage is already on the way
+        cur.init(sg.P, sg.K, (int64_t)mt * TILE, M, sg.Q, sg.K, (int64_t)nt * TILE, p.N, 0, (int)sg.K);
+        if (s > 0) cur.issue_first_leader(smem);
+        gemm_tile_run<2, 2, false>(acc, smem, cur);
+      }
+    } else {
+      for (int s = 0; s < nseg; ++s) {
+        const NoLoaders none{0, (int)p.seg[seg0 + s].K};
+        gemm_tile_run<2, 2, false>(acc, smem, none);
+      }
     }
     if (more) {
       const LoraSeg& sg = p.seg[p.job[j2].seg0];
-      TileLoaders<LORA_NI> nxt;
+      PlainTileLoaders nxt;
       nxt.init(sg.P, sg.K, (int64_t)mt2 * TILE, p.job[j2].M, sg.Q, sg.K, (int64_t)nt2 * TILE, p.N, 0, (int)sg.K);
       nxt.issue_first(smem);
     }

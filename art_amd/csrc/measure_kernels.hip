@@ -6,6 +6,7 @@
 #include "gemm_nt.hpp"
 #include "gemm_4x16.hpp"
 #include "gemm_half.hpp"
+#include "gemm_plain8.hpp"
 
 namespace artk {
 
@@ -173,9 +174,9 @@ struct LoopProbeParams {
 };
 
 template <int LOOP, int ABL>
-__global__ __launch_bounds__(LOOP == 0 || LOOP == 3 ? 512 : 256, LOOP == 4 ? 2 : 1) void loop_probe_kernel(
+__global__ __launch_bounds__(LOOP == 0 || LOOP == 3 || LOOP == 5 ? 512 : 256, LOOP == 4 ? 2 : 1) void loop_probe_kernel(
     LoopProbeParams p) {
-  constexpr int NI = LOOP == 0 || LOOP == 3 ? 2 : 4;
+  constexpr int NI = LOOP == 0 || LOOP == 3 || LOOP == 5 ? 2 : 4;
   __shared__ __attribute__((aligned(1024))) char smem[LOOP == 4 ? HALF_LDS_BYTES : GEMM_LDS_BYTES];
   const long long c0 = clock64(), w0 = wall_clock64();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -224,6 +225,56 @@ __global__ __launch_bounds__(LOOP == 0 || LOOP == 3 ? 512 : 256, LOOP == 4 ? 2 :
       nt = nt2;
     }
     if (threadIdx.x == 0 && p.cycles != nullptr && blockIdx.x < gridDim.x / 2) {
+      p.cycles[2 * blockIdx.x] = clock64() - c0;
+      p.cycles[2 * blockIdx.x + 1] = wall_clock64() - w0;
+    }
+    return;
+  }
+  if constexpr (LOOP == 5) {
+    // the 8-wave loop of gemm_plain8.hpp; ABL = 1: the whole fill of a stage right after the barrier
+    const int n_tiles = p.MT * p.NT;
+    int t = blockIdx.x, mt, nt;
+    tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt, p.group);
+    auto init = [&](PlainTileLoaders& L, int mt_, int nt_) {
+      const int fm = p.same_tile ? (int)(blockIdx.x & 7) : mt_, fn = p.same_tile ? (int)(blockIdx.x & 7) : nt_;
+      L.init(p.P, p.K, (int64_t)fm * TILE, p.M, p.Q, p.K, (int64_t)fn * TILE, p.N, 0, (int)p.K);
+    };
+    {
+      PlainTileLoaders first;
+      init(first, mt, nt);
+      first.issue_first(smem);
+    }
+    for (;;) {
+      const int t2 = t + gridDim.x;
+      const bool more = t2 < n_tiles;
+      int mt2 = 0, nt2 = 0;
+      if (more) tile_coords(xcd_remap(t2, n_tiles), p.MT, p.NT, mt2, nt2, p.group);
+      TileAcc<2> acc;
+      acc.zero();
+      {
+        PlainTileLoaders cur;
+        init(cur, mt, nt);
+        gemm_tile_run_plain8<ABL != 0>(acc, smem, cur);
+      }
+      if (more) {
+        PlainTileLoaders nx;
+        init(nx, mt2, nt2);
+        nx.issue_first(smem);
+      }
+      const int wm = wave_m<2>(wave), wn = wave_n<2>(wave);
+#pragma unroll
+      for (int ni = 0; ni < 2; ++ni) {
+        const int64_t col = (int64_t)nt * TILE + acc_col<2>(wn, ni, lane);
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+          store_block_bf16(p.out + col * p.M + (int64_t)mt * TILE + wm * 128 + mi * 32, acc.c[mi][ni], lane >> 5);
+      }
+      if (!more) break;
+      t = t2;
+      mt = mt2;
+      nt = nt2;
+    }
+    if (threadIdx.x == 0 && p.cycles != nullptr) {
       p.cycles[2 * blockIdx.x] = clock64() - c0;
       p.cycles[2 * blockIdx.x + 1] = wall_clock64() - w0;
     }
@@ -392,12 +443,13 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
   ARTK_CHECK_ARG(aligned16(P) && aligned16(Q) && aligned16(out), "pointers must be 16-byte aligned");
   ARTK_CHECK_ARG(M >= 2048 && N >= 2048 && K >= 128 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0,
                  "M and N must be multiples of 256 (at least 2048), K a multiple of 64 (at least 128)");
-  ARTK_CHECK_ARG(loop >= 0 && loop <= 4,
-                 "loop must be 0 (8-wave), 1 (4-wave 32x32x16), 2 (4-wave 16x16x32), 3 (8-wave 16x16x32) or 4 "
-                 "(256 x 128 tiles, two work-groups per CU)");
-  ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 && (ablate == 0 || loop == 2 || (loop == 3 && ablate != 3)),
+  ARTK_CHECK_ARG(loop >= 0 && loop <= 5,
+                 "loop must be 0 (8-wave), 1 (4-wave 32x32x16), 2 (4-wave 16x16x32), 3 (8-wave 16x16x32), 4 "
+                 "(256 x 128 tiles, two work-groups per CU) or 5 (8-wave, DMA issued by the first wave of each SIMD)");
+  ARTK_CHECK_ARG(ablate >= 0 && ablate <= 7 && ablate != 6 &&
+                     (ablate == 0 || loop == 2 || (loop == 3 && ablate != 3) || (loop == 5 && ablate == 1)),
                  "ablate: bits 1 (no DMA), 2 (no barrier), 4 (no LDS reads); 6 is not built (nor 3 with loop 3); only "
-                 "with loops 2 and 3");
+                 "with loops 2 and 3; with loop 5, 1 selects the whole fill right after the barrier");
   ARTK_CHECK_ARG(group >= 1 && group <= 64, "group must be in 1..64");
   LoopProbeParams p;
   p.P = P;
@@ -429,6 +481,10 @@ int32_t artk_gemm_loop_probe(const void* P, const void* Q, void* out, int64_t M,
       case 5: loop_probe_kernel<3, 5><<<grid, 512, 0, st>>>(p); break;
       default: loop_probe_kernel<3, 7><<<grid, 512, 0, st>>>(p); break;
     }
+  }
+  else if (loop == 5) {
+    if (ablate == 0) loop_probe_kernel<5, 0><<<grid, 512, 0, st>>>(p);
+    else loop_probe_kernel<5, 1><<<grid, 512, 0, st>>>(p);
   }
   else if (loop == 4) {
     const int64_t tiles2 = tiles * 2;

@@ -781,9 +781,11 @@ def lds_probe(waves: int, kind: int, reads_per_dma: int, iters: int, blocks: int
 def gemm_loop_probe(p: torch.Tensor, q: torch.Tensor, loop: int = 0, ablate: int = 0, group: int = 8,
                     same_tile: bool = False, out: Optional[torch.Tensor] = None,
                     cycles: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out bf16 [N,M] = q [N,K] @ p [M,K]^T on a chosen main loop (0: 8-wave, 1: 4-wave 32x32x16,
-    2: 4-wave 16x16x32, 3: 8-wave 16x16x32, 4: 256 x 128 tiles with two work-groups per CU), tile-order group and ablation switches (see artk_gemm_loop_probe); the result
-    is only meaningful with ablate == 0 and same_tile False."""
+    """out bf16 [N,M] = q [N,K] @ p [M,K]^T on a chosen main loop (0: 8-wave, every wave issues its own
+    DMA; 5: 8-wave, the first wave of each SIMD issues the DMA of both; 1: 4-wave 32x32x16; 2: 4-wave
+    16x16x32; 3: 8-wave 16x16x32; 4: 256 x 128 tiles with two work-groups per CU), tile-order group and
+    ablation switches (see artk_gemm_loop_probe); the result is only meaningful with same_tile False and
+    ablate == 0 (or loop 5, where ablate 1 is another correct variant)."""
     M, K = p.shape
     N = q.shape[0]
     _need(p, "p", torch.bfloat16)

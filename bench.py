@@ -1070,6 +1070,8 @@ def bench_ceiling(args, hidden=None, lm_head=None, seconds=0.6):
         cyc = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
         rows = (("8wave_32x32x16_group8", 0, 0, 8, False), ("8wave_32x32x16_group4", 0, 0, 4, False),
                 ("8wave_32x32x16_group2", 0, 0, 2, False), ("8wave_32x32x16_group16", 0, 0, 16, False),
+                ("8wave_32x32x16_first_wave_fills_group4", 5, 0, 4, False),
+                ("8wave_32x32x16_first_wave_fills_all_early_group4", 5, 1, 4, False),
                 ("4wave_32x32x16_group4", 1, 0, 4, False), ("4wave_16x16x32_group4", 2, 0, 4, False),
                 ("4wave_16x16x32_group8", 2, 0, 8, False), ("8wave_16x16x32_group4", 3, 0, 4, False),
                 ("two_workgroups_per_cu_256x128_group4", 4, 0, 4, False),

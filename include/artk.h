@@ -476,13 +476,17 @@ int32_t artk_stream_copy(const void* src, void* dst, int64_t bytes, artk_stream_
 /* artk_gemm_loop_probe: persistent plain NT GEMM out[n,m] = sum_k Q[n,k] P[m,k] (bf16 [N,M]; M, N
  *   multiples of 256, K of 64) on a choice of main loop and tile order, with switches that take
  *   parts of the loop away, to measure what each part costs under the part's power limit.
- *   loop 0: the library's 8-wave loop; 1: its 4-wave loop with pinned instruction order (both MFMA
- *   32x32x16); 2: a 4-wave loop on MFMA 16x16x32; 3: the 8-wave shape on MFMA 16x16x32; 4: 256 x 128
- *   tiles on 4 waves with a 3-stage ring of K = 32 stages, two work-groups per CU (cycles then holds
- *   the first work-group of each pair).  ablate (loops 2 and 3; results are then wrong; 6, and 3 with loop 3, are
- *   not built):
+ *   loop 0: the library's 8-wave loop as the kernels with a gathered operand run it (every wave
+ *   issues its own share of the L2 -> LDS DMA); 5: the same loop as the kernels with two plain
+ *   operands run it (the first wave of each SIMD issues the DMA of both); 1: the 4-wave loop with
+ *   pinned instruction order (all three MFMA 32x32x16); 2: a 4-wave loop on MFMA 16x16x32; 3: the
+ *   8-wave shape on MFMA 16x16x32; 4: 256 x 128 tiles on 4 waves with a 3-stage ring of K = 32
+ *   stages, two work-groups per CU (cycles then holds the first work-group of each pair).
+ *   ablate (loops 2 and 3; results are then wrong; 6, and 3 with loop 3, are not built):
  *   bit 1 no fill of the LDS stages inside the loop, bit 2 no wait for the fill and no work-group
- *   barrier, bit 4 no LDS fragment reads.  group: row-operand tiles walked per column-operand tile
+ *   barrier, bit 4 no LDS fragment reads.  With loop 5, ablate 1 instead selects the variant that
+ *   requests the whole fill of a stage right after the barrier that frees its buffer (results
+ *   correct).  group: row-operand tiles walked per column-operand tile
  *   by consecutive tile ids (the library uses 8, or 4 when the row operand streams from HBM).
  *   same_tile != 0: every work-group fetches the same 8 operand tiles whatever it computes, so every
  *   fetch hits in L2 (results wrong).  cycles int64 [work-groups][2] or NULL: core-clock cycles and

@@ -82,7 +82,7 @@ def test_lds_probe_reports_a_plausible_rate(artk_lib, gpu, waves, kind, rpd):
         ops.lds_probe(3, 0, 0, 1, 1, gpu)
 
 
-@pytest.mark.parametrize("loop,group", [(0, 8), (1, 4), (2, 8), (2, 4), (3, 4), (4, 8), (4, 4)])
+@pytest.mark.parametrize("loop,group", [(0, 8), (1, 4), (2, 8), (2, 4), (3, 4), (4, 8), (4, 4), (5, 8), (5, 4)])
 def test_gemm_loop_probe_computes_the_product(artk_lib, gpu, loop, group):
     """Without ablation switches every loop variant of the probe is a correct GEMM (fp32 matmul of the
     bf16 inputs, bf16 rounding of the result); with a switch set it still runs to completion."""
@@ -101,5 +101,8 @@ def test_gemm_loop_probe_computes_the_product(artk_lib, gpu, loop, group):
         for ablate in (1, 2, 4, 7):
             ops.gemm_loop_probe(p, q, loop=loop, ablate=ablate, group=group, same_tile=True)
         torch.cuda.synchronize()
+    if loop == 5:  # its second variant is a correct GEMM too
+        out1 = ops.gemm_loop_probe(p, q, loop=5, ablate=1, group=group)
+        assert ((out1.float() - ref).norm() / ref.norm()).item() < 4e-3
     with pytest.raises(ValueError):
         ops.gemm_loop_probe(p, q, loop=1, ablate=1)
