@@ -19,7 +19,7 @@ namespace artk {
 // Work-group shape of each GEMM kernel (see gemm_nt.hpp).
 constexpr int FWD_NI = 2;   // lm_head projection + log-sum-exp epilogue: 8 waves
 constexpr int BWD_NI = 2;   // d_hidden GEMM
-constexpr int GEMM_NI = 4;  // plain GEMM: 4 waves, pinned order (+2..4 % over the 8-wave shape)
+constexpr int GEMM_NI = 2;  // plain GEMM: 8 waves, the first wave of each SIMD issues the DMA (gemm_plain8.hpp)
 
 // ----------------------------------------------------------------------------
 // index helpers
@@ -847,6 +847,18 @@ __device__ __forceinline__ void gemm_nt_store(const TileAcc<NI>& acc, const Gemm
   const int wave = threadIdx.x >> 6;
   const int wm = wave_m<NI>(wave), wn = wave_n<NI>(wave);
   const int half = lane >> 5;
+  if (!p.out_f32 && (p.M & 7) == 0 && (int64_t)(mt + 1) * TILE <= p.M) {
+    // bf16 and all 256 rows inside: 16-byte stores (lanes l and l + 32 hold the same column and trade halves)
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+      const int64_t col = (int64_t)nt * TILE + acc_col<NI>(wn, ni, lane);
+      if (col >= p.N) continue;
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+        store_block_bf16((uint16_t*)p.out + col * p.M + (int64_t)mt * TILE + wm * 128 + mi * 32, acc.c[mi][ni], half);
+    }
+    return;
+  }
 #pragma unroll
   for (int ni = 0; ni < NI; ++ni) {
     const int64_t col = (int64_t)nt * TILE + acc_col<NI>(wn, ni, lane);
@@ -872,16 +884,42 @@ __device__ __forceinline__ void gemm_nt_store(const TileAcc<NI>& acc, const Gemm
   }
 }
 
+// Persistent: one work-group per CU walks tiles b, b + grid, ...; the next tile's first DMA stage is started
+// before the current tile is stored.
 __global__ __launch_bounds__(nthreads<GEMM_NI>()) void gemm_nt_kernel(GemmParams p) {
   __shared__ __attribute__((aligned(1024))) char smem[GEMM_LDS_BYTES];
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  int mt, nt;
-  tile_coords(id, p.MT, p.NT, mt, nt, p.MT >= 8 * p.NT ? TILE_GROUP_STREAMING : TILE_GROUP);
-  TileAcc<GEMM_NI> acc;
-  acc.zero();
-  gemm_tile_nt(acc, smem, p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0,
-               (int)p.K);
-  gemm_nt_store<GEMM_NI>(acc, p, mt, nt);
+  const int n_tiles = p.MT * p.NT;
+  const int group = p.MT >= 8 * p.NT ? TILE_GROUP_STREAMING : TILE_GROUP;
+  int t = blockIdx.x, mt, nt;
+  tile_coords(xcd_remap(t, n_tiles), p.MT, p.NT, mt, nt, group);
+  {
+    PlainTileLoaders first;
+    first.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
+    first.issue_first(smem);
+  }
+  for (;;) {
+    const int t2 = t + gridDim.x;
+    const bool more = t2 < n_tiles;
+    int mt2 = 0, nt2 = 0;
+    if (more) tile_coords(xcd_remap(t2, n_tiles), p.MT, p.NT, mt2, nt2, group);
+    TileAcc<GEMM_NI> acc;
+    acc.zero();
+    {
+      PlainTileLoaders cur;  // its first stage is already on the way
+      cur.init(p.P, p.K, (int64_t)mt * TILE, p.M, p.Q, p.K, (int64_t)nt * TILE, p.N, 0, (int)p.K);
+      gemm_tile_run_plain8<false>(acc, smem, cur);
+    }
+    if (more) {
+      PlainTileLoaders nxt;
+      nxt.init(p.P, p.K, (int64_t)mt2 * TILE, p.M, p.Q, p.K, (int64_t)nt2 * TILE, p.N, 0, (int)p.K);
+      nxt.issue_first(smem);
+    }
+    gemm_nt_store<GEMM_NI>(acc, p, mt, nt);
+    if (!more) break;
+    t = t2;
+    mt = mt2;
+    nt = nt2;
+  }
 }
 
 // ----------------------------------------------------------------------------
@@ -1464,7 +1502,8 @@ int32_t artk_gemm_nt(const void* P, const void* Q, void* out, int64_t M, int64_t
   p.MT = (int)((M + TILE - 1) / TILE);
   p.NT = (int)((N + TILE - 1) / TILE);
   p.out_f32 = out_f32;
-  gemm_nt_kernel<<<(unsigned)(p.MT * p.NT), nthreads<GEMM_NI>(), 0, (hipStream_t)stream>>>(p);
+  const int64_t n_tiles = (int64_t)p.MT * p.NT;
+  gemm_nt_kernel<<<(unsigned)(n_tiles < num_cus() ? n_tiles : num_cus()), nthreads<GEMM_NI>(), 0, (hipStream_t)stream>>>(p);
   ARTK_CHECK_LAUNCH();
   return ARTK_OK;
 }

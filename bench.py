@@ -28,7 +28,7 @@ PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E peak
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs
 # (FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size); None until
 # measured for the workload.  Source: profiles/lmhead_fwd_c3_pmc.md
-TRAFFIC_BYTES = {"c3": 1.60e10, "c1": None}  # 7.48e6 x 2 KiB fetched + 0.70e6 KiB written per forward launch
+TRAFFIC_BYTES = {"c3": 1.68e10, "c1": None}  # 7.87e6 x 2 KiB fetched + 0.70e6 KiB written per forward launch
 # moe_gemm_kernel, mean bytes per launch over the 4 launches of the step with gate|up fused (FETCH_SIZE x 2 KiB +
 # WRITE_SIZE x 1 KiB, the factors a 1 GiB copy gives): 1166 MB read + 211 MB written
 MOE_TRAFFIC_BYTES = 1.38e9
