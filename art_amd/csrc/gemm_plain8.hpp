@@ -36,7 +36,10 @@ struct PanelLoader {
     const char* p = (const char*)base + row0 * ld * 2;
     const int64_t left = nrows - row0;
     const int64_t nvalid = left >= TILE ? TILE : (left > 0 ? left : 0);
-    rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, (int)(nvalid * ld * 2), 0x00020000);
+    // (a tile spans 256 * ld * 2 bytes, which must stay below 2 GiB as for every loader here: the
+    // per-lane offsets are 32-bit)
+    const int64_t bytes = nvalid * ld * 2;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, (int)(bytes < 0x7fffffff ? bytes : 0x7fffffff), 0x00020000);
     const int r = lane >> 3, pc = lane & 7;
     voff[0] = (int)(r * ld * 2) + ((pc ^ r) << 4);  // swz(8g + r) = r ^ (g & 1)
     voff[1] = (int)(r * ld * 2) + ((pc ^ r ^ 1) << 4);
