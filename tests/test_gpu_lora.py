@@ -42,7 +42,8 @@ def run_gpu(x, W, A, B, up, scale, gpu):
 
 
 @pytest.mark.parametrize("T,n_in,n_out,r", [(512, 256, 256, 8), (300, 192, 320, 8), (256, 128, 64, 16),
-                                            (1000, 512, 576, 24)])
+                                            (1000, 512, 576, 24),
+                                            (5000, 192, 4160, 8)])  # more tiles than CUs, ragged on both sides
 def test_lora_matches_oracle(artk_lib, gpu, T, n_in, n_out, r):
     print(f"lora T={T} in={n_in} out={n_out} r={r}", flush=True)
     x, W, A, B, up = make(T, n_in, n_out, r, T + r)
